@@ -1,9 +1,11 @@
 from .registry import (ConfigError, config_from_dict, load_config, register_architecture,
                        registered_architectures)
-from .specs import (AttentionSpec, BlockSpec, GatedFeedForwardSpec, Llama3RopeScaling, ModelSpec,
-                    NormSpec, RotarySpec, Run)
+from .specs import (AttentionSpec, BlockSpec, DistanceBias, GatedDeltaSpec, GatedFeedForwardSpec, Inject,
+                    Llama3RopeScaling, ModelSpec, NormSpec, RotarySpec, Run)
 from .llama import LlamaConfiguration
+from .melizen import MelizenConfiguration
 
 __all__ = ["ConfigError", "config_from_dict", "load_config", "register_architecture",
            "registered_architectures", "AttentionSpec", "BlockSpec", "GatedFeedForwardSpec",
-           "Llama3RopeScaling", "ModelSpec", "NormSpec", "RotarySpec", "Run", "LlamaConfiguration"]
+           "Llama3RopeScaling", "ModelSpec", "NormSpec", "RotarySpec", "Run", "LlamaConfiguration", "DistanceBias", "GatedDeltaSpec", "Inject",
+           "MelizenConfiguration"]

@@ -1,5 +1,5 @@
-"""One registry from the architecture's name (``architectures[0]`` of config.json)
-to its typed configuration.
+"""One registry from the architecture's name (``architectures[0]`` of config.json, or its
+``architecture`` where a folder names one as a plain string) to its typed configuration.
 
 The reference maps an enum constant to a loader and throws for an unknown type
 (J/model/ModelType.java:24-75); here the key is the name the model folder itself
@@ -29,6 +29,8 @@ def registered_architectures():
 
 def config_from_dict(d):
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        archs = [d["architecture"]]
     if not isinstance(archs, (list, tuple)) or not archs:
         raise ConfigError("config.json: 'architectures' is missing or empty; "
                           f"registered: {registered_architectures()}")

@@ -35,10 +35,23 @@ class RotarySpec:
 
 @dataclass(frozen=True)
 class NormSpec:
+    """``x / sqrt(mean(x^2) + eps) * (weight_offset + w)``: a weight stored around zero has ``weight_offset`` 1."""
     kind: str = "rmsnorm"
     dim: int = 0
     eps: float = 1e-5
     names: dict = field(default_factory=dict)     # local tensor name -> stored name
+    weight_offset: float = 0.0
+
+
+@dataclass(frozen=True)
+class DistanceBias:
+    """A bias on the attention scores that grows with the distance: head h of H takes
+    ``slope_h * (i - j)`` off the score of query i and key j, ``slope_h = base ** (-exponent * (h + 1) / H)``."""
+    base: float = 2.0
+    exponent: float = 8.0
+
+    def slopes(self, n_heads):
+        return [self.base ** (-self.exponent * (h + 1) / n_heads) for h in range(n_heads)]
 
 
 @dataclass(frozen=True)
@@ -54,23 +67,51 @@ class AttentionSpec:
     window: Optional[int] = None      # None: every earlier key; n: the last n keys
     scale: Optional[float] = None     # None: 1/sqrt(head_dim)
     names: dict = field(default_factory=dict)
+    v_head_dim: Optional[int] = None  # the values' size; None: the keys'
+    distance_bias: Optional[DistanceBias] = None
+    sink: Optional[float] = None      # the score of a key without a value that every query sees (it takes its share
+                                      # of the softmax's weights and adds nothing); None: no such key
+    out_scale_name: Optional[str] = None   # a stored [hidden] vector that the mixer's output is multiplied by
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """The gated delta rule: per value head a matrix [key_dim, value_dim] in 32-bit that every token decays,
+    corrects towards its value along its key, and reads with its query (``parts/delta.py``). ``n_heads`` value
+    heads share ``n_kv_heads`` query/key heads; q, k and v pass a causal convolution of ``conv_taps`` taps."""
+    kind: str = "gated_delta"
+    hidden: int = 0
+    n_heads: int = 0
+    n_kv_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    conv_taps: int = 1
+    unit_eps: float = 1e-6            # inside the root when q and k are scaled to unit length
+    norm_eps: float = 1e-5            # the read-out's norm
+    names: dict = field(default_factory=dict)
+    out_scale_name: Optional[str] = None
 
 
 @dataclass(frozen=True)
 class GatedFeedForwardSpec:
-    """down(act(gate(x)) * up(x)); ``activation``: "silu" or "gelu_tanh". Names ``gate_bias`` and
-    ``up_bias`` (together) and ``down_bias`` among ``names`` add biases to the products."""
+    """down(act(gate(x)) * (up(x) + up_shift)); ``activation``: "silu", "gelu_tanh" or "quick_gelu"
+    (z * sigmoid(1.702 z)). A ``limit`` bounds the gate from above and the up value on both sides before
+    that. Names ``gate_bias`` and ``up_bias`` (together) and ``down_bias`` among ``names`` add biases to the products."""
     kind: str = "gated"
     hidden: int = 0
     intermediate: int = 0
     activation: str = "silu"
     names: dict = field(default_factory=dict)
+    limit: Optional[float] = None
+    up_shift: float = 0.0
+    out_scale_name: Optional[str] = None   # a stored [hidden] vector that the output is multiplied by
 
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """One layer: how norm, mixer and feed-forward are arranged is ``kind``."""
-    kind: str = "prenorm"             # x += mixer(norm(x)); x += ffn(norm(x))
+    """One layer: how norm, mixer and feed-forward are arranged is ``kind``. "prenorm": x += mixer(norm(x));
+    x += ffn(norm(x)). "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h) (one norm, ``ffn_norm`` is None)."""
+    kind: str = "prenorm"
     mixer_norm: object = None
     mixer: object = None
     ffn_norm: object = None
@@ -88,6 +129,17 @@ class Run:
     """
     layer: int
     reads: Optional[int] = None
+    before: Optional["Inject"] = None     # what is added to the residual rows right before this entry runs
+
+
+@dataclass(frozen=True)
+class Inject:
+    """Added to every token's residual row: the embedding's output (the rows as they were before the first
+    block) when ``embedding``, then row ``row`` of the stored table ``vector_name`` ([rows, hidden]) if named."""
+    embedding: bool = False
+    vector_name: Optional[str] = None
+    vector_rows: int = 0
+    row: int = 0
 
 
 @dataclass(frozen=True)

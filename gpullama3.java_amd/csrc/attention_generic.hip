@@ -10,6 +10,12 @@
 // values are summed with the weights (:134-144). The chunking depends on the
 // query's position alone, so a token's result is the same bit for bit whether it
 // arrives with its whole prompt or alone.
+//
+// What other decoders ask of the same loop, all optional: values of another size than the keys
+// (v_head_dim); a bias that grows with the distance, score - slopes[h] * (p - key), one slope per
+// query head; and a sink, a key that every query sees with the score `sink` and whose value is
+// zero, so that the weights of the real keys sum to less than one: exp(s_j) / (exp(sink) + sum exp(s)).
+// The sink is the running softmax's starting point (maximum = sink, sum = 1).
 #include "common.h"
 
 #define ATT_MAX_HS 256
@@ -18,8 +24,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-    int table_stride, T* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int page_size,
-    int window, float scale) {
+    int table_stride, T* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
+    int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink) {
   __shared__ float qs[ATT_MAX_HS];
   __shared__ float ps[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -30,7 +36,8 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   const T* qp = q + (long)t * q_stride + (long)h * head_dim;
   for (int i = lane; i < head_dim; i += 64) qs[i] = to_f32<T>(qp[i]);
   __syncthreads();
-  float m = -INFINITY, l = 0.f;
+  const float slope = slopes ? slopes[h] : 0.f;
+  float m = has_sink ? sink : -INFINITY, l = has_sink ? 1.f : 0.f;
   float acc[ATT_MAX_HS / 64] = {};
   for (int base = lo; base <= p; base += 64) {
     const int key = base + lane;
@@ -41,7 +48,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       const int in_page = key % page_size;
       float dot = 0.f;
       for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32<T>(kp[gl3_k_offset(in_page, i, head_dim)]), dot);
-      s = dot * scale;
+      s = dot * scale - slope * (float)(p - key);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float pe = valid ? expf(s - m_new) : 0.f;
@@ -56,29 +63,30 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     for (int j = 0; j < n_valid; ++j) {
       const int kj = base + j;
       // values lie transposed in a page: [head_dim][position in page], in tiles
-      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * head_dim;
+      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * v_head_dim;
       const int in_page = kj % page_size;
       const float w = ps[j];
 #pragma unroll
       for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
         const int i = lane + 64 * r;
-        if (i < head_dim) acc[r] = fmaf(w, to_f32<T>(vp[gl3_v_offset(i, in_page, page_size)]), acc[r]);
+        if (i < v_head_dim) acc[r] = fmaf(w, to_f32<T>(vp[gl3_v_offset(i, in_page, page_size)]), acc[r]);
       }
     }
     m = m_new;
   }
-  T* op = out + (long)t * out_stride + (long)h * head_dim;
+  T* op = out + (long)t * out_stride + (long)h * v_head_dim;
 #pragma unroll
   for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
     const int i = lane + 64 * r;
-    if (i < head_dim) op[i] = from_f32<T>(acc[r] / l);
+    if (i < v_head_dim) op[i] = from_f32<T>(acc[r] / l);
   }
 }
 
 extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k_cache, const void* v_cache, int dtype,
                                      const int* positions, const int* seq_of_token, const int* block_table,
                                      int table_stride, void* out, long out_stride, int n_tokens, int n_heads, int n_kv,
-                                     int head_dim, int page_size, int window, float scale, hipStream_t stream) {
+                                     int head_dim, int page_size, int window, float scale, int v_head_dim,
+                                     const float* slopes, int has_sink, float sink, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
               "gl3_attention_generic: null argument");
@@ -86,6 +94,8 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
               "gl3_attention_generic: %d heads over %d kv heads", n_heads, n_kv);
   GL3_REQUIRE(head_dim > 0 && head_dim <= ATT_MAX_HS, "gl3_attention_generic: head_dim %d exceeds %d", head_dim,
               ATT_MAX_HS);
+  GL3_REQUIRE(v_head_dim > 0 && v_head_dim <= ATT_MAX_HS && v_head_dim % 16 == 0,
+              "gl3_attention_generic: v_head_dim %d is not a multiple of 16 up to %d", v_head_dim, ATT_MAX_HS);
   GL3_REQUIRE(n_heads <= 65535, "gl3_attention_generic: %d heads exceed the grid", n_heads);
   GL3_REQUIRE(page_size > 0 && table_stride > 0, "gl3_attention_generic: bad paging");
   GL3_REQUIRE(page_size % 32 == 0 && head_dim % 16 == 0,
@@ -95,11 +105,13 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
   if (dtype == GL3_F32)
     attention_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, positions, seq_of_token, block_table,
-        table_stride, (float*)out, out_stride, n_heads, n_kv, head_dim, page_size, window, scale);
+        table_stride, (float*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink,
+        sink);
   else if (dtype == GL3_BF16)
     attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,
-        block_table, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, head_dim, page_size, window, scale);
+        block_table, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale,
+        slopes, has_sink, sink);
   else GL3_REQUIRE(false, "gl3_attention_generic: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;

@@ -136,7 +136,8 @@ __host__ __device__ __forceinline__ long gl3_w_offset(int order, long n, int k, 
   return gl3_packed_offset(n, k, steps);
 }
 
-enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1 };
+enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1, GL3_ACT_QUICK_GELU = 2 };
+#define GL3_ACT_KNOWN(act) ((act) >= GL3_ACT_SILU && (act) <= GL3_ACT_QUICK_GELU)
 
 template <bool FAST>
 __device__ __forceinline__ float gl3_activation(float v, int act) {
@@ -145,5 +146,21 @@ __device__ __forceinline__ float gl3_activation(float v, int act) {
     const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
     return v / (1.0f + (FAST ? __expf(-2.0f * u) : expf(-2.0f * u)));
   }
+  if (act == GL3_ACT_QUICK_GELU) {   // v * sigmoid(1.702 v), the sigmoid form of gelu
+    const float u = 1.702f * v;
+    return v / (1.0f + (FAST ? __expf(-u) : expf(-u)));
+  }
   return v / (1.0f + (FAST ? __expf(-v) : expf(-v)));
+}
+
+// The gated epilogue's rule in full: act(gate) * (up + shift), where a positive `limit` first bounds the
+// gate from above (min(gate, limit)) and the up value on both sides (clamp(up, -limit, limit)). The
+// reference's feed-forward is limit = 0 (none), shift = 0.
+template <bool FAST>
+__device__ __forceinline__ float gl3_gated(float gate, float up, int act, float limit, float shift) {
+  if (limit > 0.f) {
+    gate = fminf(gate, limit);
+    up = fminf(fmaxf(up, -limit), limit);
+  }
+  return gl3_activation<FAST>(gate, act) * (up + shift);
 }

@@ -568,3 +568,79 @@ extern "C" int gl3_decode_advance(int* token_ids, int* positions, int* kv_before
   GL3_LAUNCH_CHECK();
   return 0;
 }
+
+// ----------------------------------------------------------------- keys and values of other sizes into the cache
+// Rows of a projection [T][ld] whose columns k_off .. hold n_kv keys of head_dim and v_off .. n_kv values of
+// v_head_dim go to the token's place in its page, unrotated: what an attention without a rotation, or with values
+// of another size than its keys, writes. grid (T, 2 n_kv): key heads, then value heads.
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ rows, long ld, int k_off, int v_off,
+                                const int* __restrict__ positions, const int* __restrict__ table_rows,
+                                const int* __restrict__ block_table, int table_stride, T* __restrict__ k_cache,
+                                T* __restrict__ v_cache, int n_kv, int head_dim, int v_head_dim, int page_size) {
+  const int t = blockIdx.x, u = blockIdx.y;
+  const int pos = positions[t];
+  const long page = block_table[(long)table_rows[t] * table_stride + pos / page_size];
+  const int in_page = pos % page_size;
+  if (u < n_kv) {
+    const T* src = rows + (long)t * ld + k_off + (long)u * head_dim;
+    T* kpage = k_cache + (page * n_kv + u) * page_size * head_dim;
+    for (int i = threadIdx.x; i < head_dim; i += blockDim.x) kpage[gl3_k_offset(in_page, i, head_dim)] = src[i];
+  } else {
+    const int c = u - n_kv;
+    const T* src = rows + (long)t * ld + v_off + (long)c * v_head_dim;
+    T* vpage = v_cache + (page * n_kv + c) * page_size * v_head_dim;
+    for (int i = threadIdx.x; i < v_head_dim; i += blockDim.x) vpage[gl3_v_offset(i, in_page, page_size)] = src[i];
+  }
+}
+
+extern "C" int gl3_kv_write(const void* rows, int dtype, long ld, int k_off, int v_off, const int* positions,
+                            const int* table_rows, const int* block_table, int table_stride, void* k_cache,
+                            void* v_cache, int n_tokens, int n_kv, int head_dim, int v_head_dim, int page_size,
+                            hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(rows && positions && table_rows && block_table && k_cache && v_cache && n_tokens > 0 && n_kv > 0 &&
+                  table_stride > 0, "gl3_kv_write: bad arguments");
+  GL3_REQUIRE(page_size > 0 && page_size % 32 == 0 && head_dim > 0 && head_dim % 16 == 0 && v_head_dim > 0 &&
+                  v_head_dim % 16 == 0,
+              "gl3_kv_write: the cache lies in tiles: page_size %d must be a multiple of 32, head sizes %d and %d of 16",
+              page_size, head_dim, v_head_dim);
+  GL3_REQUIRE(k_off >= 0 && v_off >= 0 && k_off + (long)n_kv * head_dim <= ld && v_off + (long)n_kv * v_head_dim <= ld &&
+                  2 * n_kv <= 65535, "gl3_kv_write: columns %d and %d of rows of %ld", k_off, v_off, ld);
+  dim3 grid(n_tokens, 2 * n_kv), block(64);
+  if (dtype == GL3_F32)
+    kv_write_kernel<float><<<grid, block, 0, stream>>>((const float*)rows, ld, k_off, v_off, positions, table_rows,
+                                                       block_table, table_stride, (float*)k_cache, (float*)v_cache, n_kv,
+                                                       head_dim, v_head_dim, page_size);
+  else if (dtype == GL3_BF16)
+    kv_write_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)rows, ld, k_off, v_off, positions, table_rows,
+                                                        block_table, table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                                        n_kv, head_dim, v_head_dim, page_size);
+  else GL3_REQUIRE(false, "gl3_kv_write: unknown dtype %d", dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- what a decoder adds to the residual rows between blocks
+// x[t, i] += rows[t, i] (may be null: nothing) + vec[i] (may be null): a run of layers that is entered again with the
+// embedding's output added back, and a learned vector per pass.
+__global__ void residual_inject_kernel(float* __restrict__ x, const float* __restrict__ rows, const float* __restrict__ vec,
+                                       long n, int d) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = x[i];
+  if (rows) v += rows[i];
+  if (vec) v += vec[i % d];
+  x[i] = v;
+}
+
+extern "C" int gl3_residual_inject(float* x, const float* rows, const float* vec, int n_tokens, int d, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(x && n_tokens > 0 && d > 0, "gl3_residual_inject: bad arguments");
+  const long n = (long)n_tokens * d;
+  const long blocks = (n + 255) / 256;
+  GL3_REQUIRE(blocks < (1L << 31), "gl3_residual_inject: %ld elements is too many", n);
+  residual_inject_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(x, rows, vec, n, d);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

@@ -12,8 +12,10 @@
 // residual stream; the reference fuses the same, TransformerComputeKernelsLayered
 // .java:766-784), and gated: W holds [gate rows | up rows] and the kernel writes
 // act(gate) * up, act = silu as the reference's (J/inference/InferenceCore.java:158-166) or the tanh form
-// of gelu. An optional bias per output column (float; gated: the gate's, then the up's) is added to
-// the sums before anything else.
+// of gelu, or its sigmoid form, optionally with bounded gate and up values and a shifted up value (gl3_gated).
+// An optional bias per output column (float; gated: the gate's, then the up's) is added to
+// the sums before anything else; an optional factor per output column (store and add epilogues: what a
+// decoder with a learned scale per channel on a sublayer's output asks for) multiplies them after that.
 #include "common.h"
 
 #define GT 64   // tile edge
@@ -26,7 +28,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
                                                             TC* __restrict__ C, int M, int N, int K, long lda,
                                                             long ldw, long ldc, long up_offset,
                                                             const float* __restrict__ bias, int act, int w_order, int w_steps,
-                                                            const int* __restrict__ w_pos) {
+                                                            const int* __restrict__ w_pos, float act_limit, float act_shift,
+                                                            const float* __restrict__ col_scale) {
   // N is the number of output columns; for EPI_GATED the up rows of W start at
   // row `up_offset`. w_order, w_steps, w_pos: how W lies (gl3_w_offset).
   __shared__ float As[GK][GT + 1];
@@ -89,7 +92,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       if (EPI == EPI_GATED) {
         float u = accu[i][j];
         if (bias) u += bias[up_offset + n];
-        v = gl3_activation<false>(v, act) * u;
+        v = gl3_gated<false>(v, u, act, act_limit, act_shift);
+      } else if (col_scale) {
+        v *= col_scale[n];
       }
       TC* c = C + m * ldc + n;
       if (EPI == EPI_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + v);
@@ -100,31 +105,35 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 
 template <typename TA, typename TW, typename TC>
 static int launch_generic(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                          int epi, const float* bias, int act, int w_order, int w_steps, const int* w_pos, hipStream_t stream) {
+                          int epi, const float* bias, int act, int w_order, int w_steps, const int* w_pos, float act_limit,
+                          float act_shift, const float* col_scale, hipStream_t stream) {
   dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT), block(256);
   GL3_REQUIRE(grid.y <= 65535, "gl3_gemm_generic: M=%d is too large for one launch", M);
   const TA* a = (const TA*)A;
   const TW* w = (const TW*)W;
   TC* c = (TC*)C;
-  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos);
-  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos);
-  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N, bias, act, w_order, w_steps, w_pos);
+  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale);
+  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale);
+  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
 // bias (may be null): N floats (gated: 2N). act: the gated epilogue's activation (GL3_ACT_*).
+// act_limit, act_shift: the gated rule's bound and shift (gl3_gated; 0, 0: none). col_scale (may be null): N floats.
 // w_order, w_pos: how W lies (see below): as stored, or one of its copies in the matrix cores' order alone.
 extern "C" int gl3_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M,
                                 int N, int K, long lda, long ldw, long ldc, int epilogue, const float* bias, int act,
-                                int w_order, const int* w_pos, hipStream_t stream) {
+                                int w_order, const int* w_pos, float act_limit, float act_shift, const float* col_scale,
+                                hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_generic: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_generic: leading dimensions %ld %ld %ld too small", lda, ldw, ldc);
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_generic: unknown epilogue %d", epilogue);
   GL3_REQUIRE(epilogue != EPI_ADD || c_dtype == GL3_F32, "gl3_gemm_generic: the add epilogue needs a float output");
-  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_generic: unknown activation %d", act);
+  GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_generic: unknown activation %d", act);
+  GL3_REQUIRE(!col_scale || epilogue != EPI_GATED, "gl3_gemm_generic: a factor per column goes with the store and add epilogues");
   // w_order: 0: W holds the rows as stored. 1: W is the copy in the matrix operands' order (lib.tile_weight); w_pos (may be
   // null) then names each row's place in it. 2: the copy in packed strips of 8 rows (lib.tile_weight8).
   const long w_rows = epilogue == EPI_GATED ? 2L * N : N;
@@ -134,12 +143,12 @@ extern "C" int gl3_gemm_generic(const void* A, int a_dtype, const void* W, int w
   const int w_steps = w_order == 1 ? (K + 31) / 32 : (K + 63) / 64;
   const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
   switch (key) {
-    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
-    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
-    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
-    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
-    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
-    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
+    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
+    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
+    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
+    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
+    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, act_limit, act_shift, col_scale, stream);
     default:
       GL3_REQUIRE(false, "gl3_gemm_generic: unsupported dtypes A=%d W=%d C=%d", a_dtype, w_dtype, c_dtype);
   }

@@ -17,7 +17,8 @@ from . import build as _build
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}     # the gated epilogue's activation
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "quick_gelu": 2}     # the gated epilogue's activation
+FAST_ACTIVATIONS = ("silu", "gelu_tanh")     # what the matrix-core products' gated epilogues apply
 
 _lib = None
 
@@ -55,8 +56,14 @@ def _declare(lib):
         "gl3_gather_rows": [P, P, P, I, I, I, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
-        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, P],
-        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
+        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, F, F, P, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, P],
+        "gl3_kv_write": [P, I, L, I, I, P, P, P, I, P, P, I, I, I, I, I, P],
+        "gl3_residual_inject": [P, P, P, I, I, P],
+        "gl3_delta_state_floats": [I, I, I, I, I],
+        "gl3_delta_prep": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, I, L, F, F, P],
+        "gl3_delta_recurrence": [P, P, P, P, P, P, I, I, I, I, I, I, L, P],
+        "gl3_delta_gated_norm": [P, P, I, I, P, I, P, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
@@ -86,6 +93,7 @@ def _declare(lib):
         fn.argtypes = args
         fn.restype = c_int
     lib.gl3_sample_work_floats.restype = ctypes.c_long
+    lib.gl3_delta_state_floats.restype = ctypes.c_long
     lib._optional = set()
 
 
@@ -148,12 +156,15 @@ def _ptr(t):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
 
-def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who):
+def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who, v_head_dim=None):
     """Keys [pages, kv heads, page, head_dim]; values transposed [pages, kv heads, head_dim, page]; inside a
     page both lie in the kernels' tiles (``cache/layout.py``), which needs pages of a multiple of 32 positions
-    and heads of a multiple of 16 elements."""
+    and heads of a multiple of 16 elements. ``v_head_dim``: the values' size where a kernel takes another than the keys'."""
+    vd = head_dim if v_head_dim is None else v_head_dim
+    if vd % 16:
+        raise KernelError(f"{who}: values of {vd} elements are not a multiple of 16")
     if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim)
-            or tuple(v_cache.shape) != (k_cache.shape[0], n_kv, head_dim, page_size)):
+            or tuple(v_cache.shape) != (k_cache.shape[0], n_kv, vd, page_size)):
         raise KernelError(f"{who}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for kv {n_kv} "
                           f"page {page_size} hs {head_dim}")
     if page_size % 32 or head_dim % 16:
@@ -326,10 +337,12 @@ def rope_cache_write(qkv, positions, seq_of_token, block_table, cos, sin, k_cach
         page_size, int(write_kv), _stream()), "rope_cache_write")
 
 
-def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu"):
+def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu", act_limit=0.0, act_shift=0.0, col_scale=None):
     """out = a @ w.T with float multiply-adds; see gemm_generic.hip for the epilogues.
     ``a`` and ``out`` may be row-strided views (last dimension contiguous). ``bias``: float32, one
-    per row of ``w``; ``act``: the gated epilogue's activation."""
+    per row of ``w``; ``act``: the gated epilogue's activation, with ``act_limit`` (a bound on gate and up
+    values, 0: none) and ``act_shift`` (added to the up value); ``col_scale``: float32, a factor per output
+    column of the store and add epilogues, applied to the sums (and the bias) before they are stored or added."""
     _dev(a, "a", contiguous=False); _dev(w, "w"); _dev(out, "out", contiguous=False)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
@@ -339,15 +352,22 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu"):
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     order, wp, pos = _w_order(w)
+    if col_scale is not None:
+        _dev(col_scale, "col_scale", torch.float32)
+        if col_scale.shape != (N,) or epilogue == EPI_GATED:
+            raise KernelError(f"gemm_generic: a factor per column {tuple(col_scale.shape)} for {N} columns, epilogue {epilogue}")
     _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), wp, _code(w, "w"), _ptr(out), _code(out, "out"),
                                       M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue,
-                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), order, pos, _stream()),
+                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), order, pos,
+                                      float(act_limit), float(act_shift), _ptr(col_scale), _stream()),
            "gemm_generic")
 
 
 def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                      page_size, window, scale):
-    """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries."""
+                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None):
+    """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries. ``v_head_dim``: the values'
+    size where it is not the keys'; ``slopes``: float32 [H], score - slopes[h] * distance; ``sink``: the score of a
+    key without a value that every query sees (None: no such key)."""
     _dev(q, "q", contiguous=False); _dev(out, "out", contiguous=False)
     _dev(k_cache, "k_cache", q.dtype); _dev(v_cache, "v_cache", q.dtype)
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
@@ -355,15 +375,118 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     T = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim or out.dtype != q.dtype:
         raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
-    if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
+    vd = head_dim if v_head_dim is None else int(v_head_dim)
+    if out.shape != (T, n_heads * vd) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
-    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention", vd)
     if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
+    if slopes is not None:
+        _dev(slopes, "slopes", torch.float32)
+        if slopes.shape != (n_heads,):
+            raise KernelError(f"attention: {tuple(slopes.shape)} slopes for {n_heads} heads")
     _check(library().gl3_attention_generic(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
-        int(window or 0), float(scale), _stream()), "attention_generic")
+        int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0), _stream()),
+        "attention_generic")
+
+
+def kv_write(rows, k_off, v_off, positions, table_rows, block_table, k_cache, v_cache, n_kv, head_dim, v_head_dim,
+             page_size):
+    """Keys (columns ``k_off`` .. of ``rows`` [T, ld]) and values (``v_off`` ..) of the step's tokens into one
+    layer's paged cache, unrotated; the values may have another size than the keys."""
+    _dev(rows, "rows", contiguous=False); _dev(positions, "positions", torch.int32)
+    _dev(table_rows, "table_rows", torch.int32); _dev(block_table, "block_table", torch.int32)
+    _dev(k_cache, "k_cache", rows.dtype); _dev(v_cache, "v_cache", rows.dtype)
+    T = rows.shape[0]
+    if rows.dim() != 2 or rows.stride(1) != 1 or positions.numel() != T or table_rows.numel() != T or block_table.dim() != 2:
+        raise KernelError(f"kv_write: rows {tuple(rows.shape)}, {positions.numel()} positions")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "kv_write", v_head_dim)
+    if k_off < 0 or v_off < 0 or k_off + n_kv * head_dim > rows.shape[1] or v_off + n_kv * v_head_dim > rows.shape[1]:
+        raise KernelError(f"kv_write: columns {k_off} and {v_off} of rows of {rows.shape[1]}")
+    _check(library().gl3_kv_write(_ptr(rows), _code(rows, "rows"), rows.stride(0), k_off, v_off, _ptr(positions),
+                                  _ptr(table_rows), _ptr(block_table), block_table.shape[1], _ptr(k_cache), _ptr(v_cache),
+                                  T, n_kv, head_dim, v_head_dim, page_size, _stream()), "kv_write")
+
+
+def residual_inject(x, rows=None, vec=None):
+    """x += rows (float32, x's shape) + vec (float32 [d]); either may be None."""
+    _dev(x, "x", torch.float32)
+    if x.dim() != 2:
+        raise KernelError(f"residual_inject: x {tuple(x.shape)}")
+    if rows is not None:
+        _dev(rows, "rows", torch.float32)
+        if rows.shape != x.shape:
+            raise KernelError(f"residual_inject: rows {tuple(rows.shape)} for x {tuple(x.shape)}")
+    if vec is not None:
+        _dev(vec, "vec", torch.float32)
+        if vec.shape != (x.shape[1],):
+            raise KernelError(f"residual_inject: a vector {tuple(vec.shape)} for rows of {x.shape[1]}")
+    _check(library().gl3_residual_inject(_ptr(x), _ptr(rows), _ptr(vec), x.shape[0], x.shape[1], _stream()),
+           "residual_inject")
+
+
+# ------------------------------------------------------------------ the gated delta rule
+def delta_state_floats(H, G, D, Dv, taps):
+    """Floats of one sequence's state: the heads' matrices in tiles of 16 value columns, then the convolution's
+    held inputs (``delta_rule.hip``). No GPU is needed to ask."""
+    return H * (-(-Dv // 16)) * D * 16 + (2 * G * D + H * Dv) * (taps - 1)
+
+
+def _delta_common(state, cu_seqlens, slot_ids, H, G, D, Dv, taps, who):
+    _dev(state, "state", torch.float32); _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
+    B = slot_ids.numel()
+    if state.dim() != 2 or state.shape[1] < delta_state_floats(H, G, D, Dv, taps) or cu_seqlens.numel() != B + 1:
+        raise KernelError(f"{who}: state {tuple(state.shape)}, {cu_seqlens.numel()} bounds for {B} sequences")
+    return B
+
+
+def delta_prep(proj, offsets, conv_w, A_log, dt_bias, state, cu_seqlens, seq_of_token, slot_ids, act, gates,
+               H, G, D, Dv, taps, unit_eps, q_scale):
+    """The step's q, k, v after the short convolution, silu and (q, k) the scaling to unit length into ``act``
+    [T, 2 G D + H Dv], the heads' decays and write strengths into ``gates`` [T, 2 H]; then each sequence's held
+    inputs move on. ``proj`` [T, ld] float32; ``offsets``: the first columns of q, k, v, b and a in it."""
+    _dev(proj, "proj", torch.float32, contiguous=False)
+    for t, n in ((conv_w, "conv_w"), (A_log, "A_log"), (dt_bias, "dt_bias"), (act, "act"), (gates, "gates")):
+        _dev(t, n, torch.float32)
+    _dev(seq_of_token, "seq_of_token", torch.int32)
+    T = proj.shape[0]
+    C = 2 * G * D + H * Dv
+    B = _delta_common(state, cu_seqlens, slot_ids, H, G, D, Dv, taps, "delta_prep")
+    if (proj.dim() != 2 or proj.stride(1) != 1 or conv_w.shape != (C, taps) or A_log.shape != (H,) or dt_bias.shape != (H,)
+            or act.shape != (T, C) or gates.shape != (T, 2 * H) or seq_of_token.numel() != T or len(offsets) != 5):
+        raise KernelError(f"delta_prep: proj {tuple(proj.shape)}, conv {tuple(conv_w.shape)}, act {tuple(act.shape)}")
+    ends = (G * D, G * D, H * Dv, H, H)
+    if any(o < 0 or o + e > proj.shape[1] for o, e in zip(offsets, ends)):
+        raise KernelError(f"delta_prep: columns {tuple(offsets)} of rows of {proj.shape[1]}")
+    _check(library().gl3_delta_prep(_ptr(proj), _ptr(conv_w), _ptr(A_log), _ptr(dt_bias), _ptr(state), _ptr(cu_seqlens),
+                                    _ptr(seq_of_token), _ptr(slot_ids), _ptr(act), _ptr(gates), T, B, H, G, D, Dv, taps,
+                                    proj.stride(0), *[int(o) for o in offsets], state.stride(0), float(unit_eps),
+                                    float(q_scale), _stream()), "delta_prep")
+
+
+def delta_recurrence(act, gates, state, cu_seqlens, slot_ids, out, H, G, D, Dv, taps):
+    """The rule itself, token by token for every sequence of the step from the state it holds; ``out`` [T, H Dv]
+    float32 receives the read-outs."""
+    _dev(act, "act", torch.float32); _dev(gates, "gates", torch.float32); _dev(out, "out", torch.float32)
+    T = act.shape[0]
+    B = _delta_common(state, cu_seqlens, slot_ids, H, G, D, Dv, taps, "delta_recurrence")
+    if act.shape != (T, 2 * G * D + H * Dv) or gates.shape != (T, 2 * H) or out.shape != (T, H * Dv):
+        raise KernelError(f"delta_recurrence: act {tuple(act.shape)}, gates {tuple(gates.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_delta_recurrence(_ptr(act), _ptr(gates), _ptr(state), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
+                                          B, H, G, D, Dv, taps, state.stride(0), _stream()), "delta_recurrence")
+
+
+def delta_gated_norm(o, proj, off_gate, weight, out, H, Dv, eps):
+    """out[t, h] = o[t, h] / rms * weight * silu(gate[t, h]), the gate in columns ``off_gate`` .. of ``proj``."""
+    _dev(o, "o", torch.float32); _dev(proj, "proj", torch.float32, contiguous=False); _dev(weight, "weight"); _dev(out, "out")
+    T = o.shape[0]
+    if (o.shape != (T, H * Dv) or out.shape != (T, H * Dv) or weight.shape != (Dv,) or proj.dim() != 2 or proj.stride(1) != 1
+            or proj.shape[0] != T or off_gate < 0 or off_gate + H * Dv > proj.shape[1]):
+        raise KernelError(f"delta_gated_norm: o {tuple(o.shape)}, proj {tuple(proj.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_delta_gated_norm(_ptr(o), _ptr(proj), proj.stride(0), off_gate, _ptr(weight), _code(weight, "weight"),
+                                          _ptr(out), _code(out, "out"), T, H, Dv, float(eps), _stream()), "delta_gated_norm")
 
 
 def decode_advance(token_ids, positions, kv_before, sampled, history, step):

@@ -6,6 +6,11 @@ and k, cache write at the token's position, attention over positions lo..p of th
 token's own sequence, output projection added into the residual stream. The reference's
 projections have no biases; a description that names ``q_bias``, ``k_bias``, ``v_bias``
 (together) or ``o_bias`` among its tensors gets them added in the products' epilogues.
+
+What other decoders' descriptions may ask for besides: no rotation (``position`` None), values of another size than
+the keys (``v_head_dim``), a bias on the scores that grows with the distance (``distance_bias``: a slope per head), a
+sink in the softmax (``sink``), and a learned factor per channel on the output (``out_scale_name``), applied by the
+output projection's epilogue.
 """
 from __future__ import annotations
 
@@ -29,7 +34,15 @@ class GQAAttention:
         self.d, self.H, self.Kh, self.hs = spec.hidden, spec.n_heads, spec.n_kv_heads, spec.head_dim
         if self.H % self.Kh:
             raise ValueError(f"{self.H} heads are not a multiple of {self.Kh} kv heads")
+        self.vd = spec.v_head_dim if getattr(spec, "v_head_dim", None) else self.hs
         self.window = spec.window
+        self.sink = getattr(spec, "sink", None)
+        bias = getattr(spec, "distance_bias", None)
+        self._slopes_host = bias.slopes(self.H) if bias is not None else None
+        self.slopes = None
+        self.device = device
+        self.out_scale_name = getattr(spec, "out_scale_name", None)
+        self.out_scale = None
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(self.hs)
         self.position = build_part("position", spec.position, device=device) if spec.position is not None else None
         self.names = spec.names
@@ -39,14 +52,17 @@ class GQAAttention:
         self.w_qkv = self.w_q = self.w_o = self.b_qkv = self.b_o = None
 
     def tensors(self):
-        n, d, hs = self.names, self.d, self.hs
+        n, d, hs, vd = self.names, self.d, self.hs, self.vd
         out = {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
-               n["v"]: TensorSpec((self.Kh * hs, d)), n["o"]: TensorSpec((d, self.H * hs))}
+               n["v"]: TensorSpec((self.Kh * vd, d)), n["o"]: TensorSpec((d, self.H * vd))}
         if self.biased:
-            out.update({n["q_bias"]: TensorSpec((self.H * hs,), "vector"), n["k_bias"]: TensorSpec((self.Kh * hs,), "vector"),
-                        n["v_bias"]: TensorSpec((self.Kh * hs,), "vector")})
+            out.update({n["q_bias"]: TensorSpec((self.H * hs,), "vector", 0.0, 0.1),
+                        n["k_bias"]: TensorSpec((self.Kh * hs,), "vector", 0.0, 0.1),
+                        n["v_bias"]: TensorSpec((self.Kh * vd,), "vector", 0.0, 0.1)})
         if "o_bias" in n:
-            out[n["o_bias"]] = TensorSpec((d,), "vector")
+            out[n["o_bias"]] = TensorSpec((d,), "vector", 0.0, 0.1)
+        if self.out_scale_name:
+            out[self.out_scale_name] = TensorSpec((d,), "vector", 1.0, 0.1)
         return out
 
     def load(self, weights):
@@ -54,14 +70,16 @@ class GQAAttention:
         parts = [weights[n["q"]], weights[n["k"]], weights[n["v"]]]
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         self.w_qkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
-        qn, kn = self.H * self.hs, self.Kh * self.hs
+        qn, kn, vn = self.H * self.hs, self.Kh * self.hs, self.Kh * self.vd
         # the stored names stay addressable as views of the stacked matrix
         weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
             self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
         self.w_q = self.w_qkv[:qn]
         without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
+        # (the strips of the copy pair up what a rotation's end pairs up; values of another size: a plain copy)
         ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
-                                      bool(self.position is not None and self.position.adjacent)), without=without)
+                                      bool(self.position is not None and self.position.adjacent))
+                         if self.vd == self.hs else None, without=without)
         self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
         if getattr(self, "may_hold_once", False):
             # the stored order is let go where a copy in the matrix cores' order can stand for the matrix; the stored
@@ -70,29 +88,50 @@ class GQAAttention:
                 self.w_qkv, self.w_q = K.hold_once(self.w_qkv), None
                 weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
                     ops.StoredRows(self, "w_qkv", 0, qn), ops.StoredRows(self, "w_qkv", qn, qn + kn),
-                    ops.StoredRows(self, "w_qkv", qn + kn, qn + 2 * kn))
+                    ops.StoredRows(self, "w_qkv", qn + kn, qn + kn + vn))
             if ops.can_hold_once(self.w_o, without):
                 self.w_o = weights[n["o"]] = K.hold_once(self.w_o)
         if self.biased:     # the epilogues read biases as float
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
         if "o_bias" in n:
             self.b_o = weights[n["o_bias"]].float().contiguous()
+        if self.out_scale_name:
+            self.out_scale = weights[self.out_scale_name].float().contiguous()
+        if self._slopes_host is not None:
+            self.slopes = torch.tensor(self._slopes_host, dtype=torch.float64).to(torch.float32).to(self.w_qkv.device)
 
     def kv_need(self):
-        return KVNeed(self.Kh, self.hs, self.window)
+        return KVNeed(self.Kh, self.hs, self.window, v_head_dim=None if self.vd == self.hs else self.vd)
 
     def state_need(self):
         return None
 
     def forward(self, ctx, h, x, run):
-        T, H, Kh, hs = h.shape[0], self.H, self.Kh, self.hs
+        T, H, Kh, hs, vd = h.shape[0], self.H, self.Kh, self.hs, self.vd
         k_cache, v_cache = ctx.cache.layer_kv(run.kv_entry)
         table = ctx.block_table(ctx.cache.group_index(run.kv_entry))
-        q = ops.qkv_project(ctx, h, self.w_qkv, self.w_q, self.position, k_cache, v_cache, table, H, Kh, hs,
-                            self.dtype, run.writes_kv, bias=self.b_qkv)
-        att = ctx.buffer("attn_out", (T, H * hs), self.dtype)
-        ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale)
-        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx, bias=self.b_o)
+        if vd == hs:
+            q = ops.qkv_project(ctx, h, self.w_qkv, self.w_q, self.position, k_cache, v_cache, table, H, Kh, hs,
+                                self.dtype, run.writes_kv, bias=self.b_qkv)
+        else:
+            q = self._project_unequal(ctx, h, k_cache, v_cache, table, run)
+        att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
+        ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
+                      slopes=self.slopes, sink=self.sink)
+        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx, bias=self.b_o, col_scale=self.out_scale)
+
+    def _project_unequal(self, ctx, h, k_cache, v_cache, table, run):
+        """Values of another size than the keys: one product over the stacked rows, then keys and values into the
+        cache as they are (such a description has no rotation)."""
+        if self.position is not None or not run.writes_kv:
+            raise ValueError("an attention whose values have another size than its keys is built without a rotation "
+                             "and with keys and values of its own")
+        T, qn, kn, vn = h.shape[0], self.H * self.hs, self.Kh * self.hs, self.Kh * self.vd
+        qkv = ctx.buffer("qkv", (T, qn + kn + vn), self.dtype)
+        ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
+        K.kv_write(qkv, qn, qn + kn, ctx.positions, ops._table_rows(ctx), table, k_cache, v_cache, self.Kh, self.hs,
+                   self.vd, k_cache.shape[2])
+        return qkv
 
 
 register_part("mixer", "attention", GQAAttention)

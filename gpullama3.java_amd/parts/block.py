@@ -48,4 +48,41 @@ class PreNormBlock:
         return part
 
 
+class ParallelBlock:
+    """One norm whose output feeds both the mixer and the feed-forward; both add into the residual rows:
+    ``h = norm(x); x += mixer(h) + ffn(h)``. The rows are complete after the later of the two, so only that one may
+    leave what the norm that reads them next would use."""
+
+    def __init__(self, spec, dtype, device):
+        if spec.ffn_norm is not None:
+            raise ValueError("a parallel block has one norm: its description names no norm for the feed-forward")
+        self.norm = build_part("norm", spec.mixer_norm, dtype=dtype)
+        self.mixer = build_part("mixer", spec.mixer, dtype=dtype, device=device)
+        self.ffn = build_part("ffn", spec.ffn, dtype=dtype, device=device) if spec.ffn is not None else None
+
+    def parts(self):
+        return [p for p in (self.norm, self.mixer, self.ffn) if p is not None]
+
+    def cache_needs(self):
+        return self.mixer.kv_need(), self.mixer.state_need()
+
+    def first_norm(self):
+        return self.norm
+
+    def forward(self, ctx, x, run, norm_after=None):
+        h = PreNormBlock._whole_rows_for(self.norm, "takes_slices", ctx, x)(ctx, x)
+        if self.ffn is not None and isinstance(h, ops.Normed):
+            # a norm that a product was to take over is worked out from the rows when somebody asks for it; the
+            # feed-forward asks after the mixer has added to them, so it is worked out now
+            h = h.materialize()
+        # (both sublayers read h, and a product of the first must not prepare rows that are not whole yet)
+        ctx.next_norm = None if self.ffn is not None else norm_after
+        PreNormBlock._whole_rows_for(self.mixer, "adds_only", ctx, x).forward(ctx, h, x, run)
+        if self.ffn is not None:
+            ctx.next_norm = norm_after
+            PreNormBlock._whole_rows_for(self.ffn, "adds_only", ctx, x).forward(ctx, h, x)
+        ctx.next_norm = None
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)

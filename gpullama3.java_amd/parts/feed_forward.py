@@ -2,7 +2,9 @@
 stream; the reference's is silu without biases (J/inference/InferenceCore.java:158-172).
 Gate and up are one product over the two matrices stacked by rows; the activation is the
 product's epilogue, and so are biases when the description names them
-(``gate_bias``, ``up_bias``, ``down_bias`` among its tensor names)."""
+(``gate_bias``, ``up_bias``, ``down_bias`` among its tensor names). A description may bound the gate and up values
+(``limit``), shift the up value (``up_shift``) and name a learned factor per channel on the output
+(``out_scale_name``, applied by the down projection's epilogue)."""
 from __future__ import annotations
 
 import torch
@@ -23,6 +25,10 @@ class GatedFeedForward:
             raise ValueError(f"activation {spec.activation!r} is not built ({sorted(ACTIVATIONS)})")
         self.d, self.F, self.dtype, self.names = spec.hidden, spec.intermediate, dtype, spec.names
         self.act = spec.activation
+        self.limit = getattr(spec, "limit", None)
+        self.up_shift = float(getattr(spec, "up_shift", 0.0))
+        self.out_scale_name = getattr(spec, "out_scale_name", None)
+        self.out_scale = None
         self.biased = "gate_bias" in self.names
         if self.biased != ("up_bias" in self.names):
             raise ValueError("a gated feed-forward names the biases of gate and up together or neither")
@@ -37,6 +43,8 @@ class GatedFeedForward:
             out[n["up_bias"]] = TensorSpec((self.F,), "vector")
         if "down_bias" in n:
             out[n["down_bias"]] = TensorSpec((self.d,), "vector")
+        if self.out_scale_name:
+            out[self.out_scale_name] = TensorSpec((self.d,), "vector", 1.0, 0.1)
         return out
 
     def load(self, weights):
@@ -60,16 +68,21 @@ class GatedFeedForward:
             self.b_gate_up = torch.cat([weights[n["gate_bias"]].float(), weights[n["up_bias"]].float()]).contiguous()
         if "down_bias" in n:
             self.b_down = weights[n["down_bias"]].float().contiguous()
+        if self.out_scale_name:
+            self.out_scale = weights[self.out_scale_name].float().contiguous()
 
     def forward(self, ctx, h, x):
-        if self.b_gate_up is None and self.b_down is None and ops.packs_rows(ctx, h, self.w_gate_up, self.w_down, x):
+        plain = not self.limit and not self.up_shift and self.out_scale is None and self.act in K.FAST_ACTIVATIONS
+        if (plain and self.b_gate_up is None and self.b_down is None
+                and ops.packs_rows(ctx, h, self.w_gate_up, self.w_down, x)):
             act = ctx.buffer("ffn_act_packed", (-(-self.F // 64), 64, 8), self.dtype)
             ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, act=self.act, pack_out=True)
             ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, a_packed=True)
             return
         act = ctx.buffer("ffn_act", (h.shape[0], self.F), self.dtype)
-        ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, bias=self.b_gate_up, act=self.act)
-        ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, bias=self.b_down)
+        ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, bias=self.b_gate_up, act=self.act, act_limit=self.limit,
+                   act_shift=self.up_shift)
+        ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, bias=self.b_down, col_scale=self.out_scale)
 
 
 register_part("ffn", "gated", GatedFeedForward)

@@ -25,6 +25,7 @@ def expected_tensors(spec, dtype=torch.float32, device="cpu"):
         out[spec.head_bias_name] = TensorSpec((spec.vocab_size,), "vector")
     if spec.final_norm is not None:
         out.update(_norm_tensors(spec.final_norm))
+    out.update(_inject_tensors(spec))
     for b in spec.layers:
         block = build_part("block", b, dtype=dtype, device=device)
         for p in block.parts():
@@ -43,6 +44,18 @@ def _block_needs(block):
         raise ValueError("a block with several parts that keep keys, values or state must say what it needs itself "
                          "(cache_needs)")
     return (keepers[0].kv_need(), keepers[0].state_need()) if keepers else (None, None)
+
+
+def _inject_tensors(spec):
+    """The tables of vectors that entries of the run order add to the residual rows before they run."""
+    out = {}
+    for r in spec.run_order:
+        b = getattr(r, "before", None)
+        if b is not None and b.vector_name is not None:
+            if not 0 <= b.row < b.vector_rows:
+                raise ValueError(f"a run-order entry adds row {b.row} of {b.vector_name!r}, which has {b.vector_rows}")
+            out[b.vector_name] = TensorSpec((b.vector_rows, spec.hidden), "matrix")
+    return out
 
 
 def _norm_tensors(spec):
@@ -87,6 +100,7 @@ class DecoderModel:
             out[self.spec.head_bias_name] = TensorSpec((self.spec.vocab_size,), "vector")
         if self.final_norm is not None:
             out.update(self.final_norm.tensors())
+        out.update(_inject_tensors(self.spec))
         for b in self.blocks:
             for p in b.parts():
                 out.update(p.tensors())
@@ -110,6 +124,10 @@ class DecoderModel:
             self.head_bias = weights[self.spec.head_bias_name].float().contiguous()
         if self.final_norm is not None:
             self.final_norm.load(weights)
+        # what entries of the run order add to the residual rows, which are 32-bit: the vectors in 32-bit
+        self.inject_vectors = {name: weights[name].float().contiguous() for name in _inject_tensors(self.spec)}
+        self.keeps_embedding = any(getattr(r, "before", None) is not None and r.before.embedding
+                                   for r in self.spec.run_order)
         for b in self.blocks:
             for p in b.parts():
                 p.load(weights)
@@ -144,7 +162,18 @@ class DecoderModel:
         else:
             K.embed(self.embedding, ctx.token_ids, x, **around)
             ops.residual_written(ctx, x)
+        embedded = None
+        if getattr(self, "keeps_embedding", False):
+            # a later entry of the run order adds the embedding's output back: looked up once more, into rows of its own
+            embedded = ctx.buffer("embedding_output", (ctx.n_tokens, self.spec.hidden), torch.float32)
+            K.embed(self.embedding, ctx.token_ids, embedded, **around)
         for i, (run, block) in enumerate(zip(self.runs, order)):
+            before = getattr(self.spec.run_order[i], "before", None)
+            if before is not None:
+                ops.settle_residual(ctx, x)
+                vec = self.inject_vectors[before.vector_name][before.row] if before.vector_name is not None else None
+                K.residual_inject(x, embedded if before.embedding else None, vec)
+                ops.residual_written(ctx, x)
             if hasattr(block, "first_norm"):
                 block.forward(ctx, x, run, norm_after=firsts[i + 1])
             else:
@@ -159,6 +188,10 @@ class DecoderModel:
                 if ctx.pending is not None:
                     raise RuntimeError("a block left sums of a product in slices behind it")
                 ops.residual_written(ctx, x)
+            watch = getattr(ctx.engine, "after_block", None)
+            if watch is not None:          # a caller that looks at the residual rows after every entry of the run order
+                ops.settle_residual(ctx, x)
+                watch(i, x)
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:

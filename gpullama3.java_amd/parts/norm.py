@@ -1,4 +1,5 @@
-"""RMSNorm: ``w * x / sqrt(mean(x^2) + eps)`` (J/inference/InferenceCore.java:47-56)."""
+"""RMSNorm: ``w * x / sqrt(mean(x^2) + eps)`` (J/inference/InferenceCore.java:47-56). A description with a
+``weight_offset`` stores its weight around zero: the factor is ``weight_offset + w``, made once, in 32-bit, at load."""
 from __future__ import annotations
 
 import torch
@@ -18,14 +19,19 @@ class RMSNorm:
 
     def __init__(self, spec, dtype):
         self.dim, self.eps, self.dtype = spec.dim, spec.eps, dtype
+        self.offset = float(getattr(spec, "weight_offset", 0.0))
         self.name = spec.names["weight"]
         self.weight = None
 
     def tensors(self):
-        return {self.name: TensorSpec((self.dim,), "vector")}
+        # (random weights: drawn around what makes the factor 1)
+        return {self.name: TensorSpec((self.dim,), "vector", center=1.0 - self.offset if self.offset else None)}
 
     def load(self, weights):
         self.weight = weights[self.name]
+        if self.offset:
+            # the sum in 32-bit: 1 + w rounded to bfloat16 would lose most of a small w
+            self.weight = (self.weight.float() + self.offset).contiguous()
         # the kernels that prepare a folded norm's rows read the weight as float (exact for 16-bit storage)
         self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 

@@ -232,12 +232,17 @@ def packs_rows(ctx, h, w_first, w_second, x):
             and K.skinny_strip_rows(M, x.shape[1], F, EPI_ADD) == 8)
 
 
-def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_out=False, a_packed=False):
+def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_out=False, a_packed=False,
+           col_scale=None, act_limit=None, act_shift=0.0):
     """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
     residual stream. ``bias`` (float32, one per row of ``w``) is added to the sums before the
-    epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``).
+    epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``), ``act_limit`` a bound on
+    the gate (from above) and the up value (both sides) and ``act_shift`` what is added to the up value;
+    ``col_scale`` (float32, one per output column; store and add epilogues) multiplies the sums.
     ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
     disabled = _off(ctx if ctx is not None else getattr(a, "ctx", None))
+    if col_scale is not None or act_limit or act_shift or act not in K.FAST_ACTIVATIONS:
+        return _linear_with_extras(a, w, out, epilogue, ctx, bias, act, col_scale, act_limit or 0.0, act_shift)
     if pack_out:
         return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
                                   pack_out=True, whole_lines=_whole_lines(a, w, epilogue))
@@ -313,6 +318,16 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
                 residual_written(ctx, out)
             return
     K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
+    if epilogue == EPI_ADD:
+        residual_written(ctx, out)
+
+
+def _linear_with_extras(a, w, out, epilogue, ctx, bias, act, col_scale, act_limit, act_shift):
+    """Products whose epilogue applies a factor per column, a bounded or shifted gated rule, or an activation that
+    only the generic product knows."""
+    if isinstance(a, Normed):
+        a = a.materialize()
+    K.gemm_generic(a, w, out, epilogue, bias=bias, act=act, act_limit=act_limit, act_shift=act_shift, col_scale=col_scale)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
 
@@ -443,9 +458,16 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     return qkv
 
 
-def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale):
+def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale, v_head_dim=None,
+              slopes=None, sink=None):
+    """``v_head_dim``: the values' size (None: the keys'); ``slopes``: float32 [H], a bias of -slopes[h] * distance
+    on the scores; ``sink``: the score of a key without a value that every query sees (None: none)."""
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     disabled = _off(ctx)
+    plain = (v_head_dim is None or v_head_dim == head_dim) and slopes is None and sink is None
+    if not plain:
+        return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
+                                   head_dim, page, window, scale, v_head_dim=v_head_dim, slopes=slopes, sink=sink)
     if q.dtype == torch.bfloat16:
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):

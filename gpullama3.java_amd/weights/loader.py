@@ -17,8 +17,12 @@ from .safetensors_io import SafetensorsError, SafetensorsFile
 
 @dataclass(frozen=True)
 class TensorSpec:
+    """``center``, ``spread``: what the random-weights mode draws a vector around and how widely (None: around 1
+    with the spread that its caller names for norm weights)."""
     shape: tuple
     kind: str = "matrix"      # "matrix" | "vector" | "table" (integers)
+    center: float = None
+    spread: float = None
 
 
 class WeightsError(ValueError):

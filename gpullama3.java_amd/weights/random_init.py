@@ -23,15 +23,17 @@ def _generator(seed, name):
     return np.random.Generator(np.random.Philox(key=[int(seed) & (2**64 - 1), zlib.crc32(name.encode("utf-8"))]))
 
 
-def random_tensor(seed, name, shape, kind, std=0.02, norm_std=0.0, vocab=None):
-    """float32 (or int64 for tables) values of one tensor."""
+def random_tensor(seed, name, shape, kind, std=0.02, norm_std=0.0, vocab=None, center=None, spread=None):
+    """float32 (or int64 for tables) values of one tensor. ``center``, ``spread``: a vector that is not a norm's
+    weight says what it is drawn around and how widely."""
     rng = _generator(seed, name)
     if kind == "table":
         return torch.from_numpy(rng.integers(0, vocab or 2, size=shape, dtype=np.int64))
     if kind == "vector":
-        v = np.ones(shape, dtype=np.float32)
-        if norm_std:
-            v += np.float32(norm_std) * rng.standard_normal(shape, dtype=np.float32)
+        v = np.full(shape, 1.0 if center is None else center, dtype=np.float32)
+        width = norm_std if spread is None else spread
+        if width:
+            v += np.float32(width) * rng.standard_normal(shape, dtype=np.float32)
         return torch.from_numpy(v)
     out = rng.standard_normal(shape, dtype=np.float32)
     out *= np.float32(std)
@@ -59,7 +61,7 @@ def write_random_model(folder, config, seed, std=0.02, norm_std=0.0, dtype="bflo
             out_dt = vdt if ts.kind == "vector" else mdt
         items.append((name, tuple(ts.shape), out_dt,
                       (lambda name=name, ts=ts, out_dt=out_dt: random_tensor(
-                          seed, name, ts.shape, ts.kind, std, norm_std, spec.vocab_size).to(out_dt))))
+                          seed, name, ts.shape, ts.kind, std, norm_std, spec.vocab_size, ts.center, ts.spread).to(out_dt))))
     write_safetensors(os.path.join(folder, "model.safetensors"), items,
                       metadata={"format": "pt", "seed": seed, "std": std, "norm_std": norm_std})
     with open(os.path.join(folder, "config.json"), "w") as f:
