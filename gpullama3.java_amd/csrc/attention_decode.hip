@@ -53,12 +53,17 @@ extern "C" int gl3_ad_stamps(long long* out) {
 // P2: a page holds a power of two of positions (page_size == 1 << page_shift): a chunk's page and its place in it are
 // a shift and a mask. A division by a number only known at run time is some forty scalar instructions, and the
 // kernel has eight of them in front of its first loads.
-template <int HS, int NW, int CB, bool P2>
+// BIAS: a bias on the scores that grows with the distance, score - slopes[head] * (p - key), and a sink (a key
+// without a value that every query sees with the score `sink`; it joins the row sums where they are completed: here
+// with one split, in the merge kernel with several). A template parameter: the kernels without them are compiled
+// as they were.
+template <int HS, int NW, int CB, bool P2, bool BIAS = false>
 __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits) {
+    long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits,
+    const float* __restrict__ slopes, int has_sink, float sink) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
   constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
@@ -105,6 +110,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   for (int kk = 0; kk < KK; ++kk)
     qt[kk] = j < heads_here ? *(const bf16x8*)(q + (long)t * q_stride + (long)(h0 + j) * HS + kk * 32 + 8 * qd) : zero8;
 
+  const float slope = (BIAS && slopes && j < heads_here) ? slopes[h0 + j] : 0.f;
   float m_run = -INFINITY, l_run = 0.f;   // l_run: this lane's share of the row sum
   f32x4 o[DT];
 #pragma unroll
@@ -155,8 +161,9 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int ka_i = key0 + 8 * qd + v, kb_i = ka_i + 4;
-        s[v] = (ka_i >= lo && ka_i < kv_len) ? sa[v] * scale : -INFINITY;
-        s[4 + v] = (kb_i >= lo && kb_i < kv_len) ? sb[v] * scale : -INFINITY;
+        const float da = BIAS ? slope * (float)(kv_len - 1 - ka_i) : 0.f;     // (the bias: slope * distance; 4 keys on: 4 slopes less)
+        s[v] = (ka_i >= lo && ka_i < kv_len) ? sa[v] * scale - da : -INFINITY;
+        s[4 + v] = (kb_i >= lo && kb_i < kv_len) ? sb[v] * scale - (BIAS ? da - 4.f * slope : 0.f) : -INFINITY;
         mx = fmaxf(mx, fmaxf(s[v], s[4 + v]));
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -219,7 +226,9 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   float M = sm_m[0][j];
 #pragma unroll
   for (int w = 1; w < NS; ++w) M = fmaxf(M, sm_m[w][j]);
-  float f[NS], L = 0.f;
+  const bool sink_here = BIAS && has_sink && n_splits == 1;
+  if (sink_here) M = fmaxf(M, sink);
+  float f[NS], L = sink_here ? __expf(sink - M) : 0.f;
 #pragma unroll
   for (int w = 0; w < NS; ++w) {
     f[w] = sm_m[w][j] == -INFINITY ? 0.f : __expf(sm_m[w][j] - M);
@@ -255,7 +264,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
 __global__ __launch_bounds__(64) void attention_decode_merge_kernel(const float* __restrict__ part_o,
                                                                     const float* __restrict__ part_ml,
                                                                     bf16_t* __restrict__ out, long out_stride, int n_heads,
-                                                                    int head_dim, int n_splits) {
+                                                                    int head_dim, int n_splits, int has_sink, float sink) {
   const long th = blockIdx.x;   // token * n_heads + head
   const long t = th / n_heads, h = th % n_heads;
   const int lane = threadIdx.x;
@@ -270,6 +279,7 @@ __global__ __launch_bounds__(64) void attention_decode_merge_kernel(const float*
   float M = fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3]));
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) M = fmaxf(M, __shfl_xor(M, d, 64));
+  if (has_sink) M = fmaxf(M, sink);
   float f[4], L = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -278,6 +288,7 @@ __global__ __launch_bounds__(64) void attention_decode_merge_kernel(const float*
   }
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) L += __shfl_xor(L, d, 64);
+  if (has_sink) L += __expf(sink - M);
   const float* po = part_o + th * n_splits * head_dim;
   for (int d = lane; d < head_dim + lane; d += 64) {     // (every lane walks the same number of times: the factors travel between lanes)
     const bool mine = d < head_dim;
@@ -307,7 +318,8 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                                     const int* positions, const int* seq_of_token, const int* block_table,
                                     int table_stride, float* part_o, float* part_ml, long part_floats, void* out,
                                     long out_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
-                                    int window, float scale, int n_splits, hipStream_t stream) {
+                                    int window, float scale, int n_splits, const float* slopes, int has_sink, float sink,
+                                    hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && block_table && out && table_stride > 0,
               "gl3_attention_decode: null argument");
@@ -332,14 +344,21 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   // More blocks than CUs: 4 waves, so that a CU holds two blocks and the second 256 blocks do not wait for the
   // first to end (what a block does before its keys arrive is a chain of trips to memory, paid once per round).
   const bool small = blocks * n_splits > 256;
+  const bool biased = slopes != nullptr || has_sink;
 #define AD_ARGS                                                                                                       \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table,    \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, n_heads / n_kv, page_size, page_shift, window,  \
-      scale, n_splits
+      scale, n_splits, slopes, has_sink, sink
 #define GO(HS)                                                                                                        \
   do {                                                                                                                \
     constexpr int CB = HS <= 64 ? 4 : HS <= 96 ? 3 : 2;                                                               \
-    if (small && p2) attention_decode_kernel<HS, 4, CB, true><<<grid, dim3(256), 0, stream>>>(AD_ARGS);                \
+    if (biased) {                                                                                                     \
+      if (small && p2) attention_decode_kernel<HS, 4, CB, true, true><<<grid, dim3(256), 0, stream>>>(AD_ARGS);        \
+      else if (small) attention_decode_kernel<HS, 4, CB, false, true><<<grid, dim3(256), 0, stream>>>(AD_ARGS);        \
+      else if (p2) attention_decode_kernel<HS, 8, CB, true, true><<<grid, dim3(512), 0, stream>>>(AD_ARGS);            \
+      else attention_decode_kernel<HS, 8, CB, false, true><<<grid, dim3(512), 0, stream>>>(AD_ARGS);                   \
+    }                                                                                                                 \
+    else if (small && p2) attention_decode_kernel<HS, 4, CB, true><<<grid, dim3(256), 0, stream>>>(AD_ARGS);           \
     else if (small) attention_decode_kernel<HS, 4, CB, false><<<grid, dim3(256), 0, stream>>>(AD_ARGS);                \
     else if (p2) attention_decode_kernel<HS, 8, CB, true><<<grid, dim3(512), 0, stream>>>(AD_ARGS);                    \
     else attention_decode_kernel<HS, 8, CB, false><<<grid, dim3(512), 0, stream>>>(AD_ARGS);                           \
@@ -355,7 +374,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   GL3_LAUNCH_CHECK();
   if (n_splits > 1) {
     attention_decode_merge_kernel<<<dim3((unsigned)((long)n_tokens * n_heads)), dim3(64), 0, stream>>>(
-        part_o, part_ml, (bf16_t*)out, out_stride, n_heads, head_dim, n_splits);
+        part_o, part_ml, (bf16_t*)out, out_stride, n_heads, head_dim, n_splits, has_sink, sink);
     GL3_LAUNCH_CHECK();
   }
   return 0;

@@ -38,12 +38,15 @@ __device__ __forceinline__ float max_over_quarters(float x) {
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
-template <int HS, int GH>
+// BIAS (both kernels): a bias on the scores that grows with the distance, score - slopes[head] * (p - key), and a
+// sink (a key without a value that every query sees with the score `sink`: the running softmax starts from it
+// instead of from nothing). A template parameter: the kernels without them are compiled as they were.
+template <int HS, int GH, bool BIAS = false>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
   constexpr int KROW = HS + 8;            // a key row in shared memory, in elements
@@ -102,9 +105,16 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   for (int hh = 0; hh < GH; ++hh) {
     m_run[hh] = -INFINITY;
     l_run[hh] = 0.f;
+    if (BIAS && has_sink) {                     // (a lane holds its quarter's share of the row sum: the sink's 1 once a query)
+      m_run[hh] = sink * 1.4426950408889634f;
+      l_run[hh] = qd == 0 ? 1.f : 0.f;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+  float sl[GH];                                 // the heads' slopes over the scale: the scores are scaled afterwards
+#pragma unroll
+  for (int hh = 0; hh < GH; ++hh) sl[hh] = (BIAS && slopes && hh < heads_here) ? slopes[h0 + hh] / scale : 0.f;
 
   // cache -> registers -> shared memory, 16 bytes a unit: a chunk's keys are 32 consecutive rows
   // of a page, its values 32 consecutive positions of each of the HS rows of the transposed page.
@@ -161,6 +171,14 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     for (int v = 0; v < 4; ++v) {
       s[v] = sa[v];
       s[4 + v] = sb[v];
+    }
+    if (BIAS) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int k1 = key0 + 8 * qd + v;
+        s[v] = fmaf(-sl[hh], (float)(p_mine - k1), s[v]);
+        s[4 + v] = fmaf(-sl[hh], (float)(p_mine - k1 - 4), s[4 + v]);
+      }
     }
     if (masked) {                               // (the same for the whole wave: a branch around the tests, one body)
 #pragma unroll
@@ -261,12 +279,12 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 // its 16 keys a step.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int HS, int CK, int AHEAD, int OCC>
+template <int HS, int CK, int AHEAD, int OCC, bool BIAS = false>
 __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
   constexpr int NT = CK / 32;             // score tiles of a chunk of CK keys
@@ -312,6 +330,11 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     qt[kk] = q_ok ? *(const bf16x8*)(q + (long)(tok0 + qi0 + n) * q_stride + (long)head * HS + kk * 16 + 8 * h) : zero8;
 
   float m_run = -INFINITY, l_run = 0.f;
+  if (BIAS && has_sink) {                       // (two lanes share a query's row sum: the sink's 1 once)
+    m_run = sink * 1.4426950408889634f;
+    l_run = h == 0 ? 1.f : 0.f;
+  }
+  const float sl = (BIAS && slopes) ? slopes[head] / scale : 0.f;
   f32x16 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -373,6 +396,15 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
         s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qt[kk], s[t], 0, 0, 0);
       }
       if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (BIAS) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = key0 + 32 * t + 16 * (v >> 3) + 8 * h + (v & 7);
+          s[t][v] = fmaf(-sl, (float)(p_mine - key), s[t][v]);
+        }
     }
     if (masked) {                               // (the same for the whole wave: a branch around the tests, one body)
 #pragma unroll
@@ -488,7 +520,8 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
                                      const int* cu_seqlens, const int* kv_before, const int* block_table,
                                      const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
                                      int max_q_len, int n_heads, int n_kv, int head_dim, int page_size, int window,
-                                     float scale, int wide_from, hipStream_t stream) {
+                                     float scale, int wide_from, const float* slopes, int has_sink, float sink,
+                                     hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && cu_seqlens && kv_before && block_table && out,
               "gl3_attention_prefill: null argument");
@@ -510,17 +543,22 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   GL3_REQUIRE(n_seqs <= 65535 && q_blocks <= 65535, "gl3_attention_prefill: %d sequences / %d blocks of queries exceed the grid",
               n_seqs, q_blocks);
   dim3 grid((unsigned)z, n_seqs, q_blocks), block(256);
+  const bool biased = slopes != nullptr || has_sink;
   if (wide) {
+#define PF_ARGS                                                                                                     \
+  (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table,     \
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink
 #define GOW(HS, CK, AH, OCC)                                                                                        \
-  attention_prefill_wide_kernel<HS, CK, AH, OCC><<<grid, block, 0, stream>>>(                                       \
-      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
-      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+  do {                                                                                                              \
+    if (biased) attention_prefill_wide_kernel<HS, CK, AH, OCC, true><<<grid, block, 0, stream>>>(PF_ARGS);          \
+    else attention_prefill_wide_kernel<HS, CK, AH, OCC, false><<<grid, block, 0, stream>>>(PF_ARGS);                \
+  } while (0)
     // chunks of 64 keys (one barrier for twice the work, two score tiles whose sums do not wait for
     // each other) where the registers hold them and a page holds whole chunks
     const bool ck64 = page_size % 64 == 0;
     switch (head_dim) {
-      case 32: if (ck64) GOW(32, 64, 2, 3); else GOW(32, 32, 2, 3); break;
-      case 64: if (ck64) GOW(64, 64, 2, 2); else GOW(64, 32, 2, 3); break;
+      case 32: if (ck64) { GOW(32, 64, 2, 3); } else { GOW(32, 32, 2, 3); } break;
+      case 64: if (ck64) { GOW(64, 64, 2, 2); } else { GOW(64, 32, 2, 3); } break;
       case 96: GOW(96, 32, 2, 2); break;
       default: GOW(128, 32, 1, 2); break;
     }
@@ -529,9 +567,10 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
     return 0;
   }
 #define GO(HS, GH)                                                                                                  \
-  attention_prefill_kernel<HS, GH><<<grid, block, 0, stream>>>(                                                     \
-      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
-      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+  do {                                                                                                              \
+    if (biased) attention_prefill_kernel<HS, GH, true><<<grid, block, 0, stream>>>(PF_ARGS);                        \
+    else attention_prefill_kernel<HS, GH, false><<<grid, block, 0, stream>>>(PF_ARGS);                              \
+  } while (0)
   switch (head_dim) {
     case 32: GO(32, 4); break;
     case 64: GO(64, 2); break;
@@ -539,6 +578,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
     default: GO(128, 1); break;
   }
 #undef GO
+#undef PF_ARGS
   GL3_LAUNCH_CHECK();
   return 0;
 }

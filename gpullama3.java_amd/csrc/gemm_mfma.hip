@@ -26,6 +26,13 @@ enum { MF_STORE = 0, MF_ADD = 1, MF_GATED = 2 };
 #define MF_BK 64
 #define MF_LD (MF_BK + 8)   // padded row, in elements
 
+// What an epilogue may apply besides a bias: a factor per output column (store and add epilogues, after the bias),
+// and the gated rule's bound and shift (gl3_gated; 0, 0: none).
+struct MfExtras {
+  const float* col_scale;
+  float act_limit, act_shift;
+};
+
 // WM x WN waves; a wave owns (32*TM) x 64 of the tile.
 template <int EPI, typename TC, int TM, int WM, int WN, int WT = 0>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
@@ -34,7 +41,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
                                                                   int tiles_m, int tiles_n, int group_m, int k_per_slice,
                                                                   float* __restrict__ P, long p_stride, long ldp,
                                                                   const float* __restrict__ bias, int act, int w_steps,
-                                                                  const int* __restrict__ w_pos) {
+                                                                  const int* __restrict__ w_pos, MfExtras ex) {
   constexpr int NT = 64 * WM * WN;                       // threads
   constexpr int BM = 32 * TM * WM;                       // rows of a block
   constexpr int BN = 64 * WN;                            // rows of W of a block
@@ -233,7 +240,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
           if (!CHECKED || n < N) {
             float g = acc[tm][0][v], u = acc[tm][1][v];
             if (bias) { g += bias[n]; u += bias[N + n]; }
-            C[(long)m * ldc + n] = from_f32<TC>(gl3_activation<true>(g, act) * u);
+            C[(long)m * ldc + n] = from_f32<TC>(gl3_gated<true>(g, u, act, ex.act_limit, ex.act_shift));
           }
         } else {
 #pragma unroll
@@ -241,7 +248,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
             const int n = n0 + wn * 64 + tn * 32 + lr;
             if (!CHECKED || n < N) {
               TC* c = C + (long)m * ldc + n;
-              const float s = acc[tm][tn][v] + (bias ? bias[n] : 0.f);
+              float s = acc[tm][tn][v] + (bias ? bias[n] : 0.f);
+              if (ex.col_scale) s *= ex.col_scale[n];
               if (EPI == MF_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + s);
               else *c = from_f32<TC>(s);
             }
@@ -257,7 +265,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 template <int EPI, typename TC, int TM, int WM, int WN, int WT = 0>
 static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
                         int slices, float* P, long p_stride, long ldp, const float* bias, int act, int w_steps,
-                        const int* w_pos, hipStream_t stream) {
+                        const int* w_pos, MfExtras ex, hipStream_t stream) {
   const int bm = 32 * TM * WM;
   const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -272,7 +280,7 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   const int group_m = tiles_m < (bm == 256 ? 4 : 8) ? tiles_m : (bm == 256 ? 4 : 8);
   gemm_mfma_kernel<EPI, TC, TM, WM, WN, WT><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
       (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, group_m, k_per_slice, P,
-      p_stride, ldp, bias, act, w_steps, w_pos);
+      p_stride, ldp, bias, act, w_steps, w_pos, ex);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -305,10 +313,10 @@ static int choose_shape(int M, int N, int slices, bool gated) {
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
                        int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape, int w_order,
-                       const int* w_pos, hipStream_t stream) {
+                       const int* w_pos, MfExtras ex, hipStream_t stream) {
   const int w_steps = w_order == 1 ? (K + 31) / 32 : w_order == 2 ? (K + 63) / 64 : 0;
   if (shape == 0) shape = choose_shape(M, N, slices, EPI == MF_GATED);
-#define MF_ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, w_pos, stream
+#define MF_ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, w_pos, ex, stream
   if (w_order) {
     // W is one of its copies in the matrix cores' order (a weight that is held once): the three tiles that the library
     // chooses between
@@ -335,14 +343,16 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // slices > 1 (not with the gated epilogue): K is cut into that many slices; the first ends in the
 // epilogue into C, slice s > 0 stores its sums into P[s - 1] ([slices - 1][M][ldp] floats,
 // p_stride elements apart), which the caller adds to C in that order.
-// bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation.
+// bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation, with its bound
+// and shift (gl3_gated; 0, 0: none). col_scale (may be null; not with slices, not gated): N floats, a factor per column.
 // shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
 // 64 x 64; 3: 256 x 256, eight waves of 128 x 64; 4: 256 rows x 128, eight waves of 64 x 64; 5: 128 rows x 256,
 // sixteen waves of 32 x 64.
 // w_order, w_pos: how W lies (see below): as stored, or one of its copies in the matrix cores' order alone.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                              long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
-                             int act, int shape, int w_order, const int* w_pos, hipStream_t stream) {
+                             int act, int shape, int w_order, const int* w_pos, float act_limit, float act_shift,
+                             const float* col_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -359,7 +369,10 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   GL3_REQUIRE(slices == 1 || (epilogue != MF_GATED && P && ldp >= N && p_stride >= (long)(M - 1) * ldp + N),
               "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
-  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
+  GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_mfma: unknown activation %d", act);
+  GL3_REQUIRE(!col_scale || (slices == 1 && epilogue != MF_GATED),
+              "gl3_gemm_mfma: a factor per column goes with one slice of K and the store and add epilogues");
+  const MfExtras ex{col_scale, act_limit, act_shift};
   GL3_REQUIRE(shape >= 0 && shape <= 5, "gl3_gemm_mfma: unknown tile shape %d", shape);
   // w_order: 0: W holds the rows as stored. 1: W is the copy in the matrix operands' order (lib.tile_weight), w_pos (may be
   // null) naming each row's place in it. 2: the copy in packed strips of 8 rows (lib.tile_weight8).
@@ -369,7 +382,7 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
                     (w_order != 1 || (w_rows % 16 == 0 && N % 16 == 0)) && (w_order != 2 || w_rows % 8 == 0) && (w_order == 1 || !w_pos),
                 "gl3_gemm_mfma: W in order %d with K=%d (a copy's order is read over whole steps of 64), N=%d", w_order, K, N);
   }
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_order, w_pos, stream
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_order, w_pos, ex, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
     if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);

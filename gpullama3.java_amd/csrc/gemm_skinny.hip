@@ -81,6 +81,8 @@ struct SkNext {
   const float* bias;      // [N] (gated: [2N]) float; null: none
   int act;
   int pack_out;           // (store and gated epilogues, at most 8 rows) the rows go out in the packed tiles' order, see sk_packed_offset
+  const float* col_scale; // [N] float (store and add epilogues): a factor per output column on the sums and the bias; null: none
+  float act_limit, act_shift;   // the gated rule's bound and shift (gl3_gated); 0, 0: none
 };
 
 // Where element k of row m (< 8) of a step lies when the step's rows are kept in the order in which the
@@ -262,7 +264,8 @@ __device__ __forceinline__ void sk_ssq_sum(float (*sm_ssq)[64], float (&sq)[SK_S
 // token tile `mt`; a lane holds 4 columns of one token.
 struct SkPre {
   f32x4 prev;
-  f32x4 bias, bias_up;   // the biases of this lane's columns (zero without a bias)
+  f32x4 bias, bias_up;   // the biases of this lane's columns (zero without a bias); store and add epilogues with a
+                         // factor per column: bias_up holds the factors
   f32x4 next_w;     // the next norm's weight at this lane's columns
   f32x4 co, si;
   int pos;
@@ -313,6 +316,7 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
       for (int c = 0; c < 4; ++c) p.bias_up[c] = sk_ld_f32(b_buf, (live && n + c < N) ? (unsigned)(N + n + c) * 4u : SK_NOWHERE);
     }
   }
+  if (EPI != SK_QKV && EPI != SK_GATED && nx.col_scale) p.bias_up = sk_ld_4f(sk_rsrc(nx.col_scale, (long)N * 4), live, n, N);
   if (EPI == SK_ADD) {
     static_assert(EPI != SK_ADD || sizeof(TC) == 4, "the add epilogue adds into a float matrix");
     const __amdgpu_buffer_rsrc_t c_buf = sk_rsrc(C, ((long)(M - 1) * ldc + N) * 4);
@@ -377,11 +381,12 @@ __device__ __forceinline__ void sk_end_tile(f32x4 v, f32x4 up, int mt, float (*s
   }
   if (EPI != SK_QKV) {
     v += pre.bias;
-    up += pre.bias_up;
+    if (EPI == SK_GATED) up += pre.bias_up;
+    else if (nx.col_scale) v *= pre.bias_up;
   }
   if (EPI == SK_GATED) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] = gl3_activation<true>(v[c], nx.act) * up[c];
+    for (int c = 0; c < 4; ++c) v[c] = gl3_gated<true>(v[c], up[c], nx.act, nx.act_limit, nx.act_shift);
   }
   if (EPI == SK_QKV) {
     const int hs = rp.head_dim;
@@ -1393,7 +1398,8 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
                                const float* next_weight, void* xg, long ldxg, const float* bias, int act,
-                               const void* w_tiled, const void* w_tiled8, int a_packed, hipStream_t stream) {
+                               const void* w_tiled, const void* w_tiled8, int a_packed, float act_limit, float act_shift,
+                               const float* col_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -1406,8 +1412,8 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || (ssq_out && ldxg >= N)),
               "gl3_gemm_skinny: the next norm's weight and its rows come together, with the sums of squares");
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
-  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny: unknown activation %d", act);
-  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act, 0};
+  GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_skinny: unknown activation %d", act);
+  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act, 0, col_scale, act_limit, act_shift};
   GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny: a copy of W in the operands' order needs N %% 16 == 0");
   a.Wt = w_tiled;
   GL3_REQUIRE(!w_tiled8 || (N % 8 == 0 && (uintptr_t)w_tiled8 % 16 == 0), "gl3_gemm_skinny: a copy of W in the packed tiles' order needs N %% 8 == 0");
@@ -1494,7 +1500,8 @@ static int wide_strips(int N, int slices, int epilogue) {
 extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                     long ldw, long ldc, int epilogue, int slices, long slice_stride,
                                     int strips_per_block, const float* bias, int act, const float* ssq, int n_partials,
-                                    float eps, int pack_out, int w_order, hipStream_t stream) {
+                                    float eps, int pack_out, int w_order, float act_limit, float act_shift,
+                                    const float* col_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
   // w_order: 0: W holds the rows as they are stored. 1: W is the copy in the matrix operands' order (lib.tile_weight,
@@ -1529,9 +1536,10 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   GL3_REQUIRE(strips_per_block == big || strips_per_block == big / 2, "gl3_gemm_skinny_wide: %d strips per block",
               strips_per_block);
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_skinny_wide: a bias goes with one slice of K");
-  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_wide: unknown activation %d", act);
+  GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_skinny_wide: unknown activation %d", act);
+  GL3_REQUIRE(!col_scale || slices == 1, "gl3_gemm_skinny_wide: a factor per column goes with one slice of K");
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{ssq, n_partials, eps, nullptr}, nullptr, SkRope{}, stream, false};
-  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out, col_scale, act_limit, act_shift};
   a.wl = w_order;
   if (ssq)
     return strips_per_block == big ? launch_wide<1, 2, SK_GATED, bf16_t, true>(a, 1, 0)
@@ -1557,18 +1565,19 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
 extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float* ssq, int n_partials, float eps,
                                     const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                                     long ldc, int epilogue, int waves, const float* bias, int act, const void* w_tiled,
-                                    int pack_out, hipStream_t stream) {
+                                    int pack_out, float act_limit, float act_shift, const float* col_scale,
+                                    hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_norm", xg, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_norm: ldc too small");
   GL3_REQUIRE(epilogue == SK_STORE || epilogue == SK_GATED, "gl3_gemm_skinny_norm: epilogue %d", epilogue);
-  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_norm: unknown activation %d", act);
+  GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_skinny_norm: unknown activation %d", act);
   GL3_REQUIRE(!pack_out || (M <= 8 && c_dtype == GL3_BF16),
               "gl3_gemm_skinny_norm: the packed tiles' order holds at most 8 rows of bfloat16 (C then has 8 * 64 * ceil(N / 64) elements)");
   const SkNorm nrm = {ssq, n_partials, eps, rows};
   SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
-  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out, col_scale, act_limit, act_shift};
   GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny_norm: a copy of W in the operands' order needs N %% 16 == 0");
   a.Wt = w_tiled;
   const int nw = pick_waves(waves, N, K);

@@ -70,21 +70,21 @@ def _declare(lib):
         "gl3_argmax_advance": [P, L, P, P, I, I, P, P, P, P, I, P, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
-        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, I, P],
-        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, F, F, P, P],
+        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, I, F, F, P, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, F, F, P, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, I, P],
         "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, P, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P, F, F, P, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
-        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
+        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P, I, F, P],
         "gl3_scatter_i32": [P, L, P, P, I, P],
         "gl3_upload": [P, P, L, P],
         "gl3_stage_decode": [P, I, I, P, P, P, I, P, P],
         "gl3_stage_step": [P, P, P, I, P, P, P, I, P, I, I, P],
         "gl3_graph_launch": [P, P],
-        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P],
+        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P, I, F, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name, None)
@@ -197,6 +197,24 @@ def _bias(bias, n, who):
         if bias.shape != (n,):
             raise KernelError(f"{who}: bias {tuple(bias.shape)} for {n} columns")
     return _ptr(bias)
+
+
+def _col_scale(col_scale, n, epilogue, who):
+    """A factor per output column (store and add epilogues): float32 [n] on the device, or None."""
+    if col_scale is not None:
+        _dev(col_scale, "col_scale", torch.float32)
+        if col_scale.shape != (n,) or epilogue == EPI_GATED:
+            raise KernelError(f"{who}: a factor per column {tuple(col_scale.shape)} for {n} columns, epilogue {epilogue}")
+    return _ptr(col_scale)
+
+
+def _slopes(slopes, n_heads, who):
+    """A slope per query head for the bias that grows with the distance: float32 [H] on the device, or None."""
+    if slopes is not None:
+        _dev(slopes, "slopes", torch.float32)
+        if slopes.shape != (n_heads,):
+            raise KernelError(f"{who}: {tuple(slopes.shape)} slopes for {n_heads} heads")
+    return _ptr(slopes)
 
 
 def _act(act, who):
@@ -583,7 +601,7 @@ def packed_rows(n_columns, dtype, device):
 
 
 def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None,
-                bias=None, act="silu", a_packed=False):
+                bias=None, act="silu", a_packed=False, act_limit=0.0, act_shift=0.0, col_scale=None):
     """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
     [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows; with it
     ``xg`` [M, N] bfloat16 may receive ``next_weight * out``, the rows as the product after the next
@@ -616,6 +634,7 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
                                      _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _tiled8(w, rows, K), int(bool(a_packed)),
+                                     float(act_limit), float(act_shift), _col_scale(col_scale, N, epilogue, "gemm_skinny"),
                                      _stream()), "gemm_skinny")
 
 
@@ -766,7 +785,8 @@ def wide_slices(N, K):
     return max(1, min(8, 256 // -(-N // 32), K // 512))
 
 
-def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu"):
+def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu", act_limit=0.0, act_shift=0.0,
+                     col_scale=None):
     """out (=, +=, gated) a @ w.T for 17 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
     (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up; that form
     also takes 9 to 16 rows."""
@@ -787,7 +807,8 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
     _check(library().gl3_gemm_skinny_wide(_ptr(a), wp, _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,
                                           _bias(bias, wrows, "gemm_skinny_wide"), _act(act, "gemm_skinny_wide"),
-                                          None, 0, 0.0, 0, order, _stream()), "gemm_skinny_wide")
+                                          None, 0, 0.0, 0, order, float(act_limit), float(act_shift),
+                                          _col_scale(col_scale, N, epilogue, "gemm_skinny_wide"), _stream()), "gemm_skinny_wide")
 
 
 def _check_norm_args(xg, ssq, n_partials, K):
@@ -807,7 +828,7 @@ def gemm_skinny_norm_fits(xg, w, out, epilogue):
 
 
 def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0, bias=None, act="silu",
-                     pack_out=False, whole_lines=False):
+                     pack_out=False, whole_lines=False, act_limit=0.0, act_shift=0.0):
     """out (=, gated) RMSNorm(x)[rows] @ w.T, where ``xg`` = bfloat16(norm weight * x) was left by the
     kernel that completed the rows of x, together with their sums of squares as partial sums.
     ``pack_out`` (at most 8 rows, bfloat16): ``out`` is a ``packed_rows`` buffer. ``whole_lines`` (gated
@@ -840,11 +861,12 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
         return _check(library().gl3_gemm_skinny_wide(
             _ptr(xg), wp, _ptr(out), _code(out, "out"), M, N, K, xg.stride(0), w.stride(0), out.stride(0), epilogue,
             1, 0, 0, _bias(bias, wrows, "gemm_skinny_norm"), _act(act, "gemm_skinny_norm"), _ptr(ssq), n_partials,
-            float(eps), int(bool(pack_out)), order, _stream()), "gemm_skinny_wide")
+            float(eps), int(bool(pack_out)), order, float(act_limit), float(act_shift), None, _stream()), "gemm_skinny_wide")
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
         xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),
-        _act(act, "gemm_skinny_norm"), _tiled(w, wrows, K, n_out=N), int(bool(pack_out)), _stream()), "gemm_skinny_norm")
+        _act(act, "gemm_skinny_norm"), _tiled(w, wrows, K, n_out=N), int(bool(pack_out)), float(act_limit), float(act_shift),
+        None, _stream()), "gemm_skinny_norm")
 
 
 def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
@@ -956,8 +978,9 @@ def decode_splits(n_tokens, n_heads, n_kv, kv_len, head_dim=64):
 
 
 def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                     page_size, window, scale, n_splits, part_o=None, part_ml=None):
-    """One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
+                     page_size, window, scale, n_splits, part_o=None, part_ml=None, slopes=None, sink=None):
+    """``slopes`` (float32 [H]): score - slopes[h] * distance; ``sink``: the score of a key without a value that every
+    query sees (None: none). One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
     are needed when ``n_splits`` > 1 (contiguous, adjacent is not required). ``seq_of_token`` None: token t's
     pages are row t of ``block_table`` (a table of the step's own, as ``token_facts`` makes it)."""
     _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
@@ -983,7 +1006,8 @@ def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, 
     _check(library().gl3_attention_decode(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
         block_table.shape[1], _ptr(part_o), _ptr(part_ml), floats, _ptr(out), out.stride(0), T, n_heads, n_kv,
-        head_dim, page_size, int(window or 0), float(scale), n_splits, _stream()), "attention_decode")
+        head_dim, page_size, int(window or 0), float(scale), n_splits, _slopes(slopes, n_heads, "attention_decode"),
+        int(sink is not None), float(sink or 0.0), _stream()), "attention_decode")
 
 
 # ------------------------------------------------------------------ bfloat16 product for many rows
@@ -995,7 +1019,8 @@ def gemm_mfma_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="silu", shape=0):
+def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="silu", shape=0, act_limit=0.0,
+              act_shift=0.0, col_scale=None):
     """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``. With
     ``more_slices`` [S, M, N] float32 K is cut into S + 1 slices: the first goes into ``out``, the
     others' sums are stored there, for the caller to add to ``out`` in that order."""
@@ -1017,8 +1042,9 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="s
     order, wp, pos = _w_order(w)
     _check(library().gl3_gemm_mfma(_ptr(a), wp, _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                    out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp,
-                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), order, pos, _stream()),
-           "gemm_mfma")
+                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), order, pos,
+                                   float(act_limit), float(act_shift), _col_scale(col_scale, N, epilogue, "gemm_mfma"),
+                                   _stream()), "gemm_mfma")
 
 
 def mfma_slices(M, N, K):
@@ -1066,8 +1092,9 @@ def attention_prefill_fits(head_dim, n_heads, n_kv, page_size):
 
 
 def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, out, max_q_len, n_heads, n_kv,
-                      head_dim, page_size, window, scale, seq_rows=None, wide_from=0):
-    """Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
+                      head_dim, page_size, window, scale, seq_rows=None, wide_from=0, slopes=None, sink=None):
+    """``slopes`` (float32 [H]): score - slopes[h] * distance; ``sink``: the score of a key without a value that every
+    query sees (None: none). Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
     of the packed ``q`` belong to which sequence and where they sit in it. ``seq_rows`` [B] (optional)
     names each sequence's row of ``block_table``; without it sequence b reads row b. ``wide_from``: from
     how many tokens of the step's longest sequence on the kernel with 128 queries a block runs
@@ -1094,7 +1121,8 @@ def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, o
     _check(library().gl3_attention_prefill(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(cu_seqlens), _ptr(kv_before), _ptr(block_table),
         _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim,
-        page_size, int(window or 0), float(scale), int(wide_from), _stream()), "attention_prefill")
+        page_size, int(window or 0), float(scale), int(wide_from), _slopes(slopes, n_heads, "attention_prefill"),
+        int(sink is not None), float(sink or 0.0), _stream()), "attention_prefill")
 
 
 # ------------------------------------------------------------------ host to device without tensor objects

@@ -193,17 +193,18 @@ def row_chunks(M, ctx=None):
     return [(lo, min(M, lo + size)) for lo in range(0, M, size)]
 
 
-def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, act="silu"):
+def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, gate=None, col_scale=None):
     M, Kd = a.shape
     N = out.shape[1]
     if epilogue != EPI_ADD:
         for lo, hi in chunks:
-            linear(a[lo:hi], w, out[lo:hi], epilogue, ctx, bias=bias, act=act)
+            linear(a[lo:hi], w, out[lo:hi], epilogue, ctx, bias=bias, col_scale=col_scale, **(gate or {}))
         return
-    slices = K.wide_slices(N, Kd) if bias is None else 1     # (a bias is added once: no slices of K with one)
+    # (a bias is added once, a factor per column applied once: no slices of K with either)
+    slices = K.wide_slices(N, Kd) if bias is None and col_scale is None else 1
     if slices < 2:
         for lo, hi in chunks:
-            K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD, bias=bias)
+            K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD, bias=bias, col_scale=col_scale)
         return residual_written(ctx, out)
     settle_residual(ctx, out)
     part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
@@ -241,11 +242,11 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     ``col_scale`` (float32, one per output column; store and add epilogues) multiplies the sums.
     ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
     disabled = _off(ctx if ctx is not None else getattr(a, "ctx", None))
-    if col_scale is not None or act_limit or act_shift or act not in K.FAST_ACTIVATIONS:
-        return _linear_with_extras(a, w, out, epilogue, ctx, bias, act, col_scale, act_limit or 0.0, act_shift)
+    gate = dict(act=act, act_limit=act_limit or 0.0, act_shift=act_shift)      # the gated epilogue's rule
+    plain_sums = bias is None and col_scale is None       # (slices of K are added up later: nothing but sums may be in them)
     if pack_out:
-        return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
-                                  pack_out=True, whole_lines=_whole_lines(a, w, epilogue))
+        return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias,
+                                  pack_out=True, whole_lines=_whole_lines(a, w, epilogue), **gate)
     if a_packed:
         M, N = out.shape
         if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
@@ -254,32 +255,33 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
             if norm is not None:
                 ssq = ctx.ssq_buffer(N // 8)
                 K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=8, next_weight=norm.weight_f32, xg=xg, bias=bias,
-                              a_packed=True)
+                              a_packed=True, col_scale=col_scale)
                 return residual_written(ctx, out, ssq, N // 8, xg, norm)
-        K.gemm_skinny(a, w, out, epilogue, strip_rows=8, bias=bias, a_packed=True)
+        K.gemm_skinny(a, w, out, epilogue, strip_rows=8, bias=bias, a_packed=True, col_scale=col_scale)
         if epilogue == EPI_ADD:
             residual_written(ctx, out)
         return
     if isinstance(a, Normed):
-        if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
+        if ("fused" not in disabled and col_scale is None and w.dtype == torch.bfloat16
+                and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
                 and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)
                 and (_whole_lines(a, w, epilogue) or K.skinny_takes(w, out.shape[0], 16))):
-            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
-                                      whole_lines=_whole_lines(a, w, epilogue))
+            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias,
+                                      whole_lines=_whole_lines(a, w, epilogue), **gate)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         chunks = row_chunks(a.shape[0], ctx)
         if (chunks and ctx is not None and getattr(ctx, "fuse", False) and not disabled & {"wide", "fused", "skinny"}
                 and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
                 and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)      # (the head: the tiled kernel)
-                and (K.skinny_takes(w, 64, 16) or (epilogue == EPI_ADD and bias is None
+                and (K.skinny_takes(w, 64, 16) or (epilogue == EPI_ADD and plain_sums
                                                    and K.wide_slices(out.shape[1], a.shape[1]) >= 2))):
-            return _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias, act)
+            return _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias, gate, col_scale)
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
-            return K.gemm_mfma(a, w, out, epilogue, bias=bias)
-        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled))
-                and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
+            return K.gemm_mfma(a, w, out, epilogue, bias=bias, col_scale=col_scale)
+        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or (col_scale is None and _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled)))
+                and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, gate, col_scale)):
             return
         rows = K.skinny_strip_rows(a.shape[0], out.shape[1], a.shape[1], epilogue)
         if not K.skinny_takes(w, a.shape[0], rows):      # (held once: through the copy it has, if it has one for these rows)
@@ -293,16 +295,16 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
                 if norm is not None:
                     ssq = ctx.ssq_buffer(N // rows)
                     K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows, next_weight=norm.weight_f32, xg=xg,
-                                  bias=bias)
+                                  bias=bias, col_scale=col_scale)
                     return residual_written(ctx, out, ssq, N // rows, xg, norm)
-            K.gemm_skinny(a, w, out, epilogue, strip_rows=rows, bias=bias, act=act)
+            K.gemm_skinny(a, w, out, epilogue, strip_rows=rows, bias=bias, col_scale=col_scale, **gate)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return
         if "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
             M, Kd = a.shape
             shape, slices = 0, 1
-            if (epilogue == EPI_ADD and bias is None and ctx is not None and getattr(ctx, "fuse", False)
+            if (epilogue == EPI_ADD and plain_sums and ctx is not None and getattr(ctx, "fuse", False)
                     and "fused" not in disabled):
                 shape, slices = K.mfma_plan(M, out.shape[1], Kd)
             if slices > 1:
@@ -313,21 +315,11 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
                 residual_written(ctx, out)
                 ctx.pending = (out.data_ptr(), part)
                 return
-            K.gemm_mfma(a, w, out, epilogue, bias=bias, act=act, shape=shape)
+            K.gemm_mfma(a, w, out, epilogue, bias=bias, shape=shape, col_scale=col_scale, **gate)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return
-    K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
-    if epilogue == EPI_ADD:
-        residual_written(ctx, out)
-
-
-def _linear_with_extras(a, w, out, epilogue, ctx, bias, act, col_scale, act_limit, act_shift):
-    """Products whose epilogue applies a factor per column, a bounded or shifted gated rule, or an activation that
-    only the generic product knows."""
-    if isinstance(a, Normed):
-        a = a.materialize()
-    K.gemm_generic(a, w, out, epilogue, bias=bias, act=act, act_limit=act_limit, act_shift=act_shift, col_scale=col_scale)
+    K.gemm_generic(a, w, out, epilogue, bias=bias, col_scale=col_scale, **gate)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
 
@@ -355,7 +347,7 @@ def _streams_rows_for_many_strips(M, w, epilogue):
             and not K.skinny_keeps_operands(M, w.shape[1]))
 
 
-def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
+def _linear_wide(a, w, out, epilogue, ctx, bias=None, gate=None, col_scale=None):
     """Products of 17 to 64 rows where another kernel than the skinny one is faster. True when done."""
     disabled = _off(ctx)
     M, Kd = a.shape
@@ -363,17 +355,17 @@ def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
     if epilogue == EPI_GATED:
         if N < 32 * 192:          # too few blocks of two strip pairs for the chip
             return False
-        K.gemm_skinny_wide(a, w, out, epilogue, bias=bias, act=act)
+        K.gemm_skinny_wide(a, w, out, epilogue, bias=bias, **(gate or {}))
         return True
     if epilogue == EPI_STORE:
         # many columns (the head): the tiled kernel, whose blocks share their rows of a; where the weight has
         # a copy in the operands' order the skinny kernel is the faster one (64 rows: 131 against 152 us)
         if (N >= 128 * 512 and "mfma" not in disabled and getattr(w, "tiled", None) is None
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
-            K.gemm_mfma(a, w, out, epilogue, bias=bias)
+            K.gemm_mfma(a, w, out, epilogue, bias=bias, col_scale=col_scale)
             return True
         return False
-    if bias is not None:          # a bias is added once: no slices of K with one
+    if bias is not None or col_scale is not None:     # a bias is added once, a factor per column applied once: no slices of K
         return False
     # into the residual stream: K in slices, added up by the norm that follows
     slices = K.wide_slices(N, Kd)
@@ -464,11 +456,8 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
     on the scores; ``sink``: the score of a key without a value that every query sees (None: none)."""
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     disabled = _off(ctx)
-    plain = (v_head_dim is None or v_head_dim == head_dim) and slopes is None and sink is None
-    if not plain:
-        return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
-                                   head_dim, page, window, scale, v_head_dim=v_head_dim, slopes=slopes, sink=sink)
-    if q.dtype == torch.bfloat16:
+    extras = dict(slopes=slopes, sink=sink)
+    if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
             T = q.shape[0]
@@ -480,13 +469,13 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
             own = getattr(ctx, "token_tables", {}).get(block_table.data_ptr())    # (made with the step's token facts)
             if own is not None:
                 return K.attention_decode(q, k_cache, v_cache, ctx.positions, None, own, out, n_heads, n_kv, head_dim, page,
-                                          window, scale, splits, part_o, part_ml)
+                                          window, scale, splits, part_o, part_ml, **extras)
             return K.attention_decode(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads,
-                                      n_kv, head_dim, page, window, scale, splits, part_o, part_ml)
+                                      n_kv, head_dim, page, window, scale, splits, part_o, part_ml, **extras)
         if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
                 and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
             return K.attention_prefill(q, k_cache, v_cache, ctx.cu_seqlens, ctx.kv_before, block_table, out,
                                        ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
-                                       seq_rows=getattr(ctx, "seq_rows", None))
+                                       seq_rows=getattr(ctx, "seq_rows", None), **extras)
     return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
-                               head_dim, page, window, scale)
+                               head_dim, page, window, scale, v_head_dim=v_head_dim, **extras)

@@ -133,6 +133,82 @@ def test_attention_sink_takes_its_share_and_the_bias_grows_with_the_distance(dty
     np.testing.assert_allclose(got, ref, atol=1e-5 if dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("splits", [1, 3])
+@pytest.mark.parametrize("H, G, D, window", [(8, 1, 64, None), (4, 2, 32, 300), (2, 2, 96, 77), (3, 1, 128, 1000)])
+def test_decode_attention_on_the_matrix_cores_with_bias_and_sink(H, G, D, window, splits):
+    """One token per sequence against a long cache, the key range cut into splits or not: the sink joins the sums
+    once, wherever they are completed."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng(D + splits)
+    S = 1100
+    bf = lambda a: torch.tensor(np.asarray(a, np.float32)).to(torch.bfloat16).float().numpy()
+    k, v = bf(rng.standard_normal((S, G, D))), bf(rng.standard_normal((S, G, D)))
+    positions = [0, 1, 31, 32, 63, 64, 500, S - 1]
+    q = bf(rng.standard_normal((len(positions), H, D)))
+    q[2] = bf(-8.0 * k[31, [h // (H // G) for h in range(H)]])        # scores far below the sink's on a short row
+    slopes = P.head_slopes(H)
+    kc, vc, table = paged(k, v, 64, "bfloat16")
+    T = len(positions)
+    out = torch.zeros(T, H * D, dtype=torch.bfloat16, device=DEV)
+    part_o = torch.empty(T, H, splits, D, device=DEV) if splits > 1 else None
+    part_ml = torch.empty(T, H, splits, 2, device=DEV) if splits > 1 else None
+    K.attention_decode(dev(q.reshape(T, H * D), torch.bfloat16), kc, vc, i32(positions), i32([0] * T), table, out, H, G, D,
+                       64, window, 0.2, splits, part_o, part_ml, slopes=dev(slopes), sink=0.0)
+    ref = plain_attention_at(q, k, v, positions, window, 0.2, slopes, 0.0)
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(T, H, D), ref, atol=2e-2)
+    K.attention_decode(dev(q.reshape(T, H * D), torch.bfloat16), kc, vc, i32(positions), i32([0] * T), table, out, H, G, D,
+                       64, window, 0.2, splits, part_o, part_ml, slopes=None, sink=-2.0)
+    ref = plain_attention_at(q, k, v, positions, window, 0.2, None, -2.0)
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(T, H, D), ref, atol=2e-2)
+
+
+@pytest.mark.parametrize("wide_from", [1, 10 ** 6])
+@pytest.mark.parametrize("H, G, D, window", [(8, 1, 64, 100), (4, 4, 32, None), (2, 1, 96, 70), (2, 2, 128, 130)])
+def test_prompt_attention_on_the_matrix_cores_with_bias_and_sink(H, G, D, window, wide_from):
+    """Both kernels for prompts (64 and 128 queries a block) over two sequences, one of which goes on from keys it
+    holds already; a marked key just inside the window of the last query, one just outside."""
+    from gpullama3_java_amd.csrc import lib as K
+    rng = np.random.default_rng(D)
+    bf = lambda a: torch.tensor(np.asarray(a, np.float32)).to(torch.bfloat16).float().numpy()
+    S0, S1, before1 = 200, 330, 150                 # sequence 1 brings 180 tokens after 150 that it holds
+    ks = [bf(0.3 * rng.standard_normal((S, G, D))) for S in (S0, S1)]
+    vs = [bf(rng.standard_normal((S, G, D))) for S in (S0, S1)]
+    qs = [bf(rng.standard_normal((S0, H, D))), bf(rng.standard_normal((S1 - before1, H, D)))]
+    if window:
+        for kk, vv, qq, last in ((ks[0], vs[0], qs[0], S0 - 1), (ks[1], vs[1], qs[1], S1 - 1)):
+            for col, j in ((0, last - window + 1), (1, last - window)):
+                if j >= 0:
+                    kk[j] = 0.0
+                    kk[j, :, col] = 8.0
+                    vv[j] = 0.0
+                    vv[j, :, col] = 5.0
+            qq[-1, :, :2] = 8.0
+    page = 64
+    n0, n1 = -(-S0 // page), -(-S1 // page)
+    from gpullama3_java_amd.cache.layout import tile_keys, tile_values
+    kc = np.zeros((1 + n0 + n1, G, page, D), np.float32)
+    vc = np.zeros((1 + n0 + n1, G, D, page), np.float32)
+    table = np.zeros((2, max(n0, n1)), np.int32)
+    table[0, :n0] = np.arange(1, 1 + n0)
+    table[1, :n1] = np.arange(1 + n0, 1 + n0 + n1)[::-1]          # (pages in another order than the positions)
+    for b, (kk, vv) in enumerate(zip(ks, vs)):
+        for j in range(len(kk)):
+            kc[table[b, j // page], :, j % page] = kk[j]
+            vc[table[b, j // page], :, :, j % page] = vv[j]
+    T = S0 + S1 - before1
+    out = torch.zeros(T, H * D, dtype=torch.bfloat16, device=DEV)
+    slopes = P.head_slopes(H)
+    K.attention_prefill(dev(np.concatenate(qs).reshape(T, H * D), torch.bfloat16), dev(tile_keys(kc), torch.bfloat16),
+                        dev(tile_values(vc), torch.bfloat16), i32([0, S0, T]), i32([0, before1]), i32(table), out,
+                        max(S0, S1 - before1), H, G, D, page, window, 0.2, wide_from=wide_from, slopes=dev(slopes), sink=0.0)
+    ref = np.concatenate([P.sink_attention(qs[0], ks[0], vs[0], 0.2, window, slopes, 0.0, 0),
+                          P.sink_attention(qs[1], ks[1], vs[1], 0.2, window, slopes, 0.0, before1)])
+    got = out.float().cpu().numpy().reshape(T, H, D)
+    np.testing.assert_allclose(got, ref, atol=3e-2)
+    if window:
+        assert got[-1, H - 1, 0] > 2.0 and abs(got[-1, :, 1]).max() < 1.0      # (the last head: the smallest slope)
+
+
 # ----------------------------------------------------------------- the delta rule's kernels
 def delta_kernels(proj, shape, conv_w, A_log, dt_bias, norm_w, state, cuts, slot, eps, dtype="float32"):
     """The three launches over one sequence cut at ``cuts``; returns the normalised, gated read-outs [T, H Dv]."""
