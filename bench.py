@@ -17,6 +17,12 @@ Two further workloads with lines of the same form:
     step (timed as the prefill), then --steps decode steps (default 128); the bytes of a step are the
     weights once and the cache at the lengths the sequences really have at that step.
   * the Llama-3.1-8B pair: ``--shape 8b --batch 64 --prompt-len 1024 --prefill-len 8192 --points ""``.
+
+``--arch melizen`` measures another decoder of the library instead, beside Llama layers of equal size on the same
+machine: a Melizen model (windowed attention with a distance bias and a sink in every other layer, a gated delta
+rule in the others, one norm a layer, a bounded gated feed-forward) with the width, feed-forward size, head sizes,
+vocabulary and layer count of ``--shape`` (``--layers`` for fewer), random weights. Its line carries prefill and
+decode throughput of both and their ratio; the default run and its line are not touched by it.
 """
 import argparse
 import json
@@ -101,6 +107,8 @@ def main():
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
+    ap.add_argument("--arch", default="llama", choices=["llama", "melizen"],
+                    help="melizen: a Melizen model of the shape's sizes beside Llama layers of equal size (a line of its own form)")
     ap.add_argument("--without", default="", help="names of fast paths to switch off for a comparison on the same machine, "
                     "comma-separated (parts/ops.py: tiled, packed, fused, wide, ...); the line then says so in `config`")
     args = ap.parse_args()
@@ -111,6 +119,9 @@ def main():
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
+
+    if args.arch == "melizen":
+        return melizen_beside_llama(args)
 
     import numpy as np
     import torch
@@ -295,6 +306,102 @@ def unequal8(args, eng, cfg, rng, shape_name, shape, esize, short, sync):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
         "points": {},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def melizen_config(shape, layers, window=1024):
+    """A Melizen model with the sizes of a Llama shape: attention layers with the shape's heads (values of the keys'
+    size) and a window, delta layers with as many value heads of the same size over the shape's kv heads, the
+    shape's feed-forward in every layer."""
+    d, F = shape["hidden_size"], shape["intermediate_size"]
+    H, G, hs = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    mlp = {"kind": "dense", "ff": F, "limit": 7.0}
+    attn = {"type": "attention", "mlp": mlp,
+            "mixer": {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5, "mask": {"size": window}}}
+    delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "conv": 4}}
+    return {"architecture": "Melizen", "vocab": shape["vocab_size"], "width": d, "max_positions": shape["max_position_embeddings"],
+            "norm": {"eps": 1e-5}, "layers": [attn if i % 2 == 0 else delta for i in range(layers)]}
+
+
+def melizen_beside_llama(args):
+    """Prefill of one prompt and decode steps at --batch for a Melizen model and for Llama layers of equal size,
+    one after the other on the same machine."""
+    import numpy as np
+    import torch
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.engine import Engine
+
+    shape_name, shape = SHAPES[args.shape]
+    layers = args.layers or shape["num_hidden_layers"]
+    K, W, B = args.steps, args.warmup, args.batch
+    prompt_len, prefill_len = args.prompt_len, args.prefill_len
+    per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    configs = {"melizen": g.config_from_dict(melizen_config(shape, layers)),
+               "llama": g.config_from_dict({**shape, "num_hidden_layers": layers})}
+    results = {}
+    for name, cfg in configs.items():
+        tmp = tempfile.mkdtemp(prefix="gl3-bench-")
+        try:
+            g.write_random_model(tmp, cfg, args.seed, norm_std=0.02)
+            eng = Engine.from_folder(tmp, dtype=args.dtype, max_tokens=max(B * per_seq, prefill_len + 64), n_slots=B,
+                                     without=args.without)
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+        rng = np.random.default_rng(args.seed)
+        V = eng.spec.vocab_size
+
+        def prefill_once():
+            s = eng.take_slot()
+            toks = rng.integers(0, V, prefill_len).tolist()
+            torch.cuda.synchronize(); t = time.perf_counter()
+            eng.step([(s, toks)])
+            torch.cuda.synchronize(); dt = time.perf_counter() - t
+            eng.give_back_slot(s)
+            return dt
+        prefill_once()
+        prefill_s = min(prefill_once() for _ in range(3))
+        slots = [eng.take_slot() for _ in range(B)]
+        for lo in range(0, B, 8):
+            eng.step([(s, rng.integers(0, V, prompt_len).tolist()) for s in slots[lo:lo + 8]], want="none")
+        temps, tops = [0.0] * B, [1.0] * B
+        toks = rng.integers(0, V, B).tolist()
+        run = eng.decode_run_length
+
+        def steps(toks, n):
+            while n > 0:
+                m = min(run, n)
+                if m > 1:
+                    toks = eng.decode_run(list(zip(slots, toks)), m, temps, tops, [[0.0] * B] * m)[-1]
+                else:
+                    toks = eng.sample(eng.step([(s, [t]) for s, t in zip(slots, toks)]), temps, tops, [0.0] * B)
+                n -= m
+            return toks
+        toks = steps(toks, W)
+        torch.cuda.synchronize(); t = time.perf_counter()
+        steps(toks, K)
+        torch.cuda.synchronize(); dt = time.perf_counter() - t
+        results[name] = {"prefill_ms": round(prefill_s * 1e3, 3), "prefill_tok_s": round(prefill_len / prefill_s, 1),
+                         "decode_ms_per_step": round(dt / K * 1e3, 4), "decode_tok_s": round(B * K / dt, 1)}
+        print(f"[bench] {name}: prefill {prefill_len} tokens {prefill_s * 1e3:.2f} ms, decode B={B} {dt / K * 1e3:.3f} ms/step",
+              file=sys.stderr, flush=True)
+        del eng
+        torch.cuda.empty_cache()
+    m, l = results["melizen"], results["llama"]
+    line = {
+        "metric": f"decode tok/s at batch {B}, Melizen model of the {shape_name}'s sizes ({prompt_len}-token prompts)",
+        "value": m["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": m["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: random N(0,0.02) weights, uniform random token ids",
+        "config": {"model": f"Melizen, sizes of the {shape_name}", "layers": layers, "global_batch": B,
+                   "seq_len": shape["max_position_embeddings"], "prompt_len": prompt_len, "prefill_len": prefill_len,
+                   "attention_window": 1024, "parallelism": "single GPU", "sampling": "greedy on device",
+                   **({"without": args.without} if args.without else {})},
+        "melizen": m, "llama_of_equal_size": l,
+        "melizen_over_llama": {"prefill_time": round(m["prefill_ms"] / l["prefill_ms"], 3),
+                               "decode_step_time": round(m["decode_ms_per_step"] / l["decode_ms_per_step"], 3)},
     }
     print(json.dumps(line))
     return 0

@@ -14,9 +14,9 @@
 // The tokens of a step are packed, sequence after sequence (cu_seqlens); each sequence is walked token by token from
 // the state that earlier steps left, so a result does not depend on how the tokens were cut into steps.
 //
-// Three launches: delta_prep (convolution, silu, unit length, decay and strength; then the convolution's new
-// state), delta_recurrence (the rule itself), delta_gated_norm (each head's read-out divided by its root mean
-// square, times a weight shared by the heads, times silu of a gate).
+// Two entry points: delta_prep (convolution, silu, unit length, decay and strength; then the convolution's new
+// state) and delta_recurrence (the rule itself, then each head's read-out divided by its root mean square, times a
+// weight shared by the heads, times silu of a gate).
 #include "common.h"
 
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
@@ -93,81 +93,166 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(const float* __re
   }
 }
 
-// grid (ceil(Dv / 16), H, B), one wave: lane (r, c) holds rows r, r + 4, ... of column c of the tile. RPL: rows a lane.
-template <int RPL>
-__global__ __launch_bounds__(64) void delta_recurrence_kernel(const float* __restrict__ act, const float* __restrict__ gates,
-                                                              float* __restrict__ state, const int* __restrict__ cu_seqlens,
-                                                              const int* __restrict__ slot_ids, float* __restrict__ out,
-                                                              DeltaShape s) {
-  const int ct = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int lane = threadIdx.x, r = lane >> 4, c = lane & 15;
-  const int j = ct * 16 + c;
-  const bool valid = j < s.Dv;
-  const int D = s.D, H = s.H;
-  const int C = 2 * s.G * D + H * s.Dv;
+// The rule itself and the read-out's norm. grid (H, B), a block of ceil(Dv / 16) waves: wave w owns the 16 value
+// columns 16 w .. of head h's matrix, lane (r, c) of it the rows r, r + 4, ... of column c (RPL rows a lane), so a
+// token costs a lane RPL multiply-adds for each of S^T k, the update and S^T q, and the sums over the four lanes of
+// a column are two lane swaps each (no trip through shared memory). The tokens' operands (k, q, v, decay,
+// strength) come in chunks of DR_CHUNK tokens through shared memory, the next chunk's loads on their way while
+// the current chunk is worked on: what a token waits for is its own chain of multiply-adds, not memory.
+// After the last token the block divides each of its tokens' read-outs (which it wrote to `o` itself) by their
+// root mean square over the head and applies the weight and the gate: y = o / rms * w * silu(gate).
+#define DR_CHUNK 16   // the most tokens a chunk; the launcher takes fewer where keys and values are long
+#define DR_NLD 8       // loads a thread has on their way for the next chunk
+
+__device__ __forceinline__ float dr_sum4(float p) {   // the sum over lanes l, l ^ 16, l ^ 32, l ^ 48
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(p), __float_as_uint(p), false, false);
+  p = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(p), __float_as_uint(p), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <int RPL, typename TO, int MAXT>
+__global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
+    const float* __restrict__ act, const float* __restrict__ gates, float* __restrict__ state,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids, float* __restrict__ o,
+    const float* __restrict__ proj, int ldp, int off_gate, const float* __restrict__ norm_w, TO* __restrict__ y,
+    float eps, DeltaShape s, int chunk, int norm_here) {
+  extern __shared__ __attribute__((aligned(16))) float dr_lds[];   // two buffers of chunk * per_token floats
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane >> 4, c = lane & 15;
+  const int D = s.D, H = s.H, Dv = s.Dv;
+  const int j = wave * 16 + c;
+  const bool valid = j < Dv;
+  const int C = 2 * s.G * D + H * Dv;
   const int kvh = h / (H / s.G);
   const int first = cu_seqlens[b], last = cu_seqlens[b + 1];
   if (last <= first) return;
-  const int CT = (s.Dv + 15) / 16;
-  float* tile = state + (long)slot_ids[b] * s.state_stride + ((long)(h * CT + ct) * D) * 16;
+  const int CT = (Dv + 15) / 16;
+  const bool owner = wave < CT;       // (a block may have more waves than tiles of columns: they only help to load)
+  float* tile = state + (long)slot_ids[b] * s.state_stride + ((long)(h * CT + (owner ? wave : 0)) * D) * 16;
   float S[RPL];
 #pragma unroll
   for (int ii = 0; ii < RPL; ++ii) {
     const int i = r + 4 * ii;
-    S[ii] = i < D ? tile[(long)i * 16 + c] : 0.f;
+    S[ii] = (owner && i < D) ? tile[(long)i * 16 + c] : 0.f;
   }
-  const long q_at = (long)kvh * D, k_at = (long)s.G * D + (long)kvh * D, v_at = 2L * s.G * D + (long)h * s.Dv + (valid ? j : 0);
-  float kr[RPL], qr[RPL], v, g, beta;
-  auto fetch = [&](int t) {
-    const float* a = act + (long)t * C;
+  // A token's operands in a chunk's buffer: q | k | v [Dv] | decay, strength, where q and k lie as the lanes read
+  // them: row r + 4 ii at [r][ii], RPL places a lane (rows beyond D stay zero), so a lane's share is 16-byte reads.
+  const int per_src = 2 * D + Dv + 2;                           // what a token brings
+  const int per_token = 8 * RPL + ((Dv + 2 + 3) & ~3);          // what it takes in the buffer
+  const int n_src = chunk * per_src;
+  const long q_at = (long)kvh * D, k_at = (long)s.G * D + (long)kvh * D, v_at = 2L * s.G * D + (long)h * Dv;
+  const int threads = blockDim.x;
+  for (int e = tid; e < 2 * chunk * per_token; e += threads) dr_lds[e] = 0.f;
+  __syncthreads();
+  float held[DR_NLD];
+  auto ask = [&](int t0) {
 #pragma unroll
-    for (int ii = 0; ii < RPL; ++ii) {
-      const int i = r + 4 * ii;
-      kr[ii] = i < D ? a[k_at + i] : 0.f;
-      qr[ii] = i < D ? a[q_at + i] : 0.f;
+    for (int n = 0; n < DR_NLD; ++n) {
+      const int e = tid + n * threads;
+      const int tt = e / per_src, f = e - tt * per_src, t = t0 + tt;
+      const float* p = act;
+      if (e < n_src && t < last) {
+        if (f < D) p = act + (long)t * C + q_at + f;
+        else if (f < 2 * D) p = act + (long)t * C + k_at + (f - D);
+        else if (f < 2 * D + Dv) p = act + (long)t * C + v_at + (f - 2 * D);
+        else p = gates + (long)t * 2 * H + (long)(f - 2 * D - Dv) * H + h;
+      }
+      held[n] = *p;
     }
-    v = a[v_at];
-    g = gates[(long)t * 2 * H + h];
-    beta = gates[(long)t * 2 * H + H + h];
   };
-  fetch(first);
-  for (int t = first; t < last; ++t) {
-    float kc[RPL], qc[RPL];
+  auto put = [&](int buf) {
 #pragma unroll
-    for (int ii = 0; ii < RPL; ++ii) { kc[ii] = kr[ii]; qc[ii] = qr[ii]; }
-    const float vc = v, gc = g, bc = beta;
-    if (t + 1 < last) fetch(t + 1);          // the next token's operands travel while this one is worked on
-    float part = 0.f;
-#pragma unroll
-    for (int ii = 0; ii < RPL; ++ii) {
-      S[ii] *= gc;
-      part = fmaf(S[ii], kc[ii], part);
+    for (int n = 0; n < DR_NLD; ++n) {
+      const int e = tid + n * threads;
+      if (e < n_src) {
+        const int tt = e / per_src, f = e - tt * per_src;
+        int at;
+        if (f < 2 * D) {
+          const int which = f >= D, i = f - which * D;
+          at = which * 4 * RPL + (i & 3) * RPL + (i >> 2);
+        } else {
+          at = 8 * RPL + (f - 2 * D);
+        }
+        dr_lds[(buf * chunk + tt) * per_token + at] = held[n];
+      }
     }
-    part += __shfl_xor(part, 16, 64);
-    part += __shfl_xor(part, 32, 64);
-    const float uu = bc * (vc - part);
-    float o = 0.f;
+  };
+  ask(first);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = first; t0 < last; t0 += chunk) {
+    const bool more = t0 + chunk < last;
+    if (more) ask(t0 + chunk);
+    const int n_here = min(chunk, last - t0);
+    for (int tt = 0; tt < n_here; ++tt) {
+      const float* op = dr_lds + (buf * chunk + tt) * per_token;
+      const float g = op[8 * RPL + Dv], beta = op[8 * RPL + Dv + 1];
+      const float v = valid ? op[8 * RPL + j] : 0.f;
+      float kc[RPL], qc[RPL];
 #pragma unroll
-    for (int ii = 0; ii < RPL; ++ii) {
-      S[ii] = fmaf(kc[ii], uu, S[ii]);
-      o = fmaf(S[ii], qc[ii], o);
+      for (int ii = 0; ii < RPL; ii += 4) {
+        const f4 q4 = *(const f4*)(op + r * RPL + ii), k4 = *(const f4*)(op + 4 * RPL + r * RPL + ii);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) { qc[ii + x] = q4[x]; kc[ii + x] = k4[x]; }
+      }
+      float p4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ii = 0; ii < RPL; ++ii) {
+        S[ii] *= g;
+        p4[ii & 3] = fmaf(S[ii], kc[ii], p4[ii & 3]);
+      }
+      const float part = dr_sum4((p4[0] + p4[1]) + (p4[2] + p4[3]));
+      const float uu = beta * (v - part);
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ii = 0; ii < RPL; ++ii) {
+        S[ii] = fmaf(kc[ii], uu, S[ii]);
+        o4[ii & 3] = fmaf(S[ii], qc[ii], o4[ii & 3]);
+      }
+      const float read = dr_sum4((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      if (r == 0 && valid) o[(long)(t0 + tt) * H * Dv + (long)h * Dv + j] = read;
     }
-    o += __shfl_xor(o, 16, 64);
-    o += __shfl_xor(o, 32, 64);
-    if (r == 0 && valid) out[(long)t * H * s.Dv + (long)h * s.Dv + j] = o;
+    if (more) put(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
   }
 #pragma unroll
   for (int ii = 0; ii < RPL; ++ii) {
     const int i = r + 4 * ii;
-    if (i < D) tile[(long)i * 16 + c] = S[ii];
+    if (owner && i < D) tile[(long)i * 16 + c] = S[ii];
+  }
+  // (steps of many tokens a sequence: a launch of its own, with a wave to every token and head, normalises them)
+  if (!norm_here) return;
+  // the read-outs of this head are all this block's own stores: made visible to its other waves, then normalised
+  __threadfence_block();
+  __syncthreads();
+  const int n_waves = threads >> 6;
+  for (int t = first + wave; t < last; t += n_waves) {
+    const float* orow = o + ((long)t * H + h) * Dv;
+    const float* grow = proj + (long)t * ldp + off_gate + (long)h * Dv;
+    float ss = 0.f;
+    for (int e = lane; e < Dv; e += 64) {
+      const float x = orow[e];
+      ss = fmaf(x, x, ss);
+    }
+    ss = wave_sum(ss);
+    const float f = 1.0f / sqrtf(ss / (float)Dv + eps);
+    TO* dst = y + ((long)t * H + h) * Dv;
+    for (int e = lane; e < Dv; e += 64) {
+      const float z = grow[e];
+      dst[e] = from_f32<TO>(orow[e] * f * norm_w[e] * (z * dr_sigmoid(z)));
+    }
   }
 }
 
-// grid (T, H), one wave: out[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :])
-template <typename TW, typename TO>
+// grid (T, H), one wave: y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :])
+template <typename TO>
 __global__ __launch_bounds__(64) void delta_gated_norm_kernel(const float* __restrict__ o, const float* __restrict__ proj,
-                                                              int ldp, int off_gate, const TW* __restrict__ w,
-                                                              TO* __restrict__ out, int H, int Dv, float eps) {
+                                                              int ldp, int off_gate, const float* __restrict__ w,
+                                                              TO* __restrict__ y, int H, int Dv, float eps) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + ((long)t * H + h) * Dv;
   const float* grow = proj + (long)t * ldp + off_gate + (long)h * Dv;
@@ -175,10 +260,10 @@ __global__ __launch_bounds__(64) void delta_gated_norm_kernel(const float* __res
   for (int e = lane; e < Dv; e += 64) ss = fmaf(orow[e], orow[e], ss);
   ss = wave_sum(ss);
   const float f = 1.0f / sqrtf(ss / (float)Dv + eps);
-  TO* dst = out + ((long)t * H + h) * Dv;
+  TO* dst = y + ((long)t * H + h) * Dv;
   for (int e = lane; e < Dv; e += 64) {
     const float z = grow[e];
-    dst[e] = from_f32<TO>(orow[e] * f * to_f32<TW>(w[e]) * (z * dr_sigmoid(z)));
+    dst[e] = from_f32<TO>(orow[e] * f * w[e] * (z * dr_sigmoid(z)));
   }
 }
 
@@ -224,44 +309,74 @@ extern "C" int gl3_delta_prep(const float* proj, const float* conv_w, const floa
   return 0;
 }
 
-// act [T][C], gates [T][2 H] as gl3_delta_prep left them; out [T][H Dv] float.
+// act [T][C], gates [T][2 H] as gl3_delta_prep left them. o [T][H Dv] float receives the raw read-outs (scratch);
+// y [T][H Dv] (float or bfloat16) the read-outs divided by their root mean square over each head, times norm_w [Dv]
+// (float), times silu of the gate, whose H Dv columns start at off_gate of proj [T][ldp] (float).
 extern "C" int gl3_delta_recurrence(const float* act, const float* gates, float* state, const int* cu_seqlens,
-                                    const int* slot_ids, float* out, int B, int H, int G, int D, int Dv, int taps,
-                                    long state_stride, hipStream_t stream) {
-  if (B == 0) return 0;
-  GL3_REQUIRE(act && gates && state && cu_seqlens && slot_ids && out && B > 0, "gl3_delta_recurrence: bad arguments");
+                                    const int* slot_ids, float* o, const float* proj, int ldp, int off_gate,
+                                    const float* norm_w, void* y, int y_dtype, float eps, int T, int B, int H, int G, int D,
+                                    int Dv, int taps, long state_stride, hipStream_t stream) {
+  if (B == 0 || T == 0) return 0;
+  GL3_REQUIRE(act && gates && state && cu_seqlens && slot_ids && o && proj && norm_w && y && B > 0,
+              "gl3_delta_recurrence: bad arguments");
   DeltaShape s;
   if (delta_shape(s, H, G, D, Dv, taps, 1 << 30, 0, 0, 0, 0, 0, state_stride)) return -1;
   GL3_REQUIRE(H <= 65535 && B <= 65535, "gl3_delta_recurrence: too many heads or sequences for the grid");
-  dim3 grid((Dv + 15) / 16, H, B), block(64);
+  GL3_REQUIRE(Dv <= 256, "gl3_delta_recurrence: values of %d elements: a block holds up to 256 columns", Dv);
+  GL3_REQUIRE(off_gate >= 0 && off_gate + H * Dv <= ldp, "gl3_delta_recurrence: the gate's columns %d .. of rows of %d", off_gate, ldp);
+  GL3_REQUIRE(y_dtype == GL3_F32 || y_dtype == GL3_BF16, "gl3_delta_recurrence: unknown dtype %d", y_dtype);
+  // as many waves as the columns need, and as the loads of a chunk of operands need (DR_NLD a thread)
+  // (fewer tokens a chunk where that keeps the block at the waves its columns need, or at four)
+  const int col_waves = (Dv + 15) / 16;
+  int chunk = DR_CHUNK, waves = col_waves;
+  for (;; chunk /= 2) {
+    waves = col_waves;
+    while (waves * 64 * DR_NLD < chunk * (2 * D + Dv + 2)) ++waves;
+    if (waves <= (col_waves > 4 ? col_waves : 4) || chunk == 1) break;
+  }
+  GL3_REQUIRE(waves <= 16, "gl3_delta_recurrence: keys of %d with values of %d need more than a block's threads", D, Dv);
+  dim3 grid(H, B), block(waves * 64);
+  // the read-outs' norm: by the block that made them where a sequence brings few tokens (a decode step), else by a
+  // launch of its own with a wave to every token and head (a block's few waves would walk a prompt's tokens one by one)
+  const int norm_here = T <= 4 * B;
   const int rows = (D + 3) / 4;
-#define GO(R) delta_recurrence_kernel<R><<<grid, block, 0, stream>>>(act, gates, state, cu_seqlens, slot_ids, out, s)
-  if (rows <= 4) GO(4);
-  else if (rows <= 8) GO(8);
-  else if (rows <= 16) GO(16);
-  else if (rows <= 24) GO(24);
-  else if (rows <= 32) GO(32);
-  else if (rows <= 48) GO(48);
-  else GO(64);
+  const int rpl = rows <= 4 ? 4 : rows <= 8 ? 8 : rows <= 16 ? 16 : rows <= 24 ? 24 : rows <= 32 ? 32 : rows <= 48 ? 48 : 64;
+  const size_t lds = 2 * (size_t)chunk * (8 * rpl + ((Dv + 2 + 3) & ~3)) * sizeof(float);
+  GL3_REQUIRE(lds <= 64 * 1024, "gl3_delta_recurrence: a chunk's operands of %zu bytes exceed shared memory", lds);
+#define GO3(R, TO, MAXT)                                                                                                \
+  delta_recurrence_kernel<R, TO, MAXT><<<grid, block, lds, stream>>>(act, gates, state, cu_seqlens, slot_ids, o, proj, ldp, \
+                                                                     off_gate, norm_w, (TO*)y, eps, s, chunk, norm_here)
+#define GO2(R, TO)                                                             \
+  do {                                                                         \
+    if (waves <= 4) GO3(R, TO, 256);                                           \
+    else if (waves <= 8) GO3(R, TO, 512);                                      \
+    else GO3(R, TO, 1024);                                                     \
+  } while (0)
+#define GO(R)                                                                  \
+  do {                                                                         \
+    if (y_dtype == GL3_F32) GO2(R, float);                                     \
+    else GO2(R, bf16_t);                                                       \
+  } while (0)
+  switch (rpl) {
+    case 4: GO(4); break;
+    case 8: GO(8); break;
+    case 16: GO(16); break;
+    case 24: GO(24); break;
+    case 32: GO(32); break;
+    case 48: GO(48); break;
+    default: GO(64); break;
+  }
 #undef GO
+#undef GO2
+#undef GO3
   GL3_LAUNCH_CHECK();
-  return 0;
-}
-
-// o [T][H Dv] float; proj [T][ldp] float with the gate's H Dv columns from off_gate on; w [Dv]; out [T][H Dv].
-extern "C" int gl3_delta_gated_norm(const float* o, const float* proj, int ldp, int off_gate, const void* w, int w_dtype,
-                                    void* out, int out_dtype, int T, int H, int Dv, float eps, hipStream_t stream) {
-  if (T == 0) return 0;
-  GL3_REQUIRE(o && proj && w && out && T > 0 && H > 0 && H <= 65535 && Dv > 0 && off_gate >= 0 && off_gate + H * Dv <= ldp,
-              "gl3_delta_gated_norm: bad arguments");
-  dim3 grid(T, H), block(64);
-#define GO(TW, TO) delta_gated_norm_kernel<TW, TO><<<grid, block, 0, stream>>>(o, proj, ldp, off_gate, (const TW*)w, (TO*)out, H, Dv, eps)
-  if (w_dtype == GL3_F32 && out_dtype == GL3_F32) GO(float, float);
-  else if (w_dtype == GL3_F32 && out_dtype == GL3_BF16) GO(float, bf16_t);
-  else if (w_dtype == GL3_BF16 && out_dtype == GL3_F32) GO(bf16_t, float);
-  else if (w_dtype == GL3_BF16 && out_dtype == GL3_BF16) GO(bf16_t, bf16_t);
-  else GL3_REQUIRE(false, "gl3_delta_gated_norm: unknown dtypes %d %d", w_dtype, out_dtype);
-#undef GO
+  if (!norm_here) {
+    GL3_REQUIRE(T <= 2147483647 / 64, "gl3_delta_recurrence: %d tokens exceed the grid", T);
+    if (y_dtype == GL3_F32)
+      delta_gated_norm_kernel<float><<<dim3(T, H), dim3(64), 0, stream>>>(o, proj, ldp, off_gate, norm_w, (float*)y, H, Dv, eps);
+    else
+      delta_gated_norm_kernel<bf16_t><<<dim3(T, H), dim3(64), 0, stream>>>(o, proj, ldp, off_gate, norm_w, (bf16_t*)y, H, Dv, eps);
+  }
   GL3_LAUNCH_CHECK();
   return 0;
 }

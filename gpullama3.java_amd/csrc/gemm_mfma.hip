@@ -231,7 +231,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 #pragma unroll
           for (int tn = 0; tn < 2; ++tn) {
             const int n = n0 + wn * 64 + tn * 32 + lr;
-            if (!CHECKED || n < N) P[(long)(slice - 1) * p_stride + (long)m * ldp + n] = acc[tm][tn][v];
+            if (!CHECKED || n < N)
+              P[(long)(slice - 1) * p_stride + (long)m * ldp + n] = ex.col_scale ? acc[tm][tn][v] * ex.col_scale[n] : acc[tm][tn][v];
           }
           continue;
         }
@@ -344,7 +345,8 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // epilogue into C, slice s > 0 stores its sums into P[s - 1] ([slices - 1][M][ldp] floats,
 // p_stride elements apart), which the caller adds to C in that order.
 // bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation, with its bound
-// and shift (gl3_gated; 0, 0: none). col_scale (may be null; not with slices, not gated): N floats, a factor per column.
+// and shift (gl3_gated; 0, 0: none). col_scale (may be null; not gated): N floats, a factor per column (every slice's sums
+// are multiplied, so the caller adds up scaled sums).
 // shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
 // 64 x 64; 3: 256 x 256, eight waves of 128 x 64; 4: 256 rows x 128, eight waves of 64 x 64; 5: 128 rows x 256,
 // sixteen waves of 32 x 64.
@@ -370,8 +372,7 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
               "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
   GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_mfma: unknown activation %d", act);
-  GL3_REQUIRE(!col_scale || (slices == 1 && epilogue != MF_GATED),
-              "gl3_gemm_mfma: a factor per column goes with one slice of K and the store and add epilogues");
+  GL3_REQUIRE(!col_scale || epilogue != MF_GATED, "gl3_gemm_mfma: a factor per column goes with the store and add epilogues");
   const MfExtras ex{col_scale, act_limit, act_shift};
   GL3_REQUIRE(shape >= 0 && shape <= 5, "gl3_gemm_mfma: unknown tile shape %d", shape);
   // w_order: 0: W holds the rows as stored. 1: W is the copy in the matrix operands' order (lib.tile_weight), w_pos (may be

@@ -1537,7 +1537,6 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
               strips_per_block);
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_skinny_wide: a bias goes with one slice of K");
   GL3_REQUIRE(GL3_ACT_KNOWN(act), "gl3_gemm_skinny_wide: unknown activation %d", act);
-  GL3_REQUIRE(!col_scale || slices == 1, "gl3_gemm_skinny_wide: a factor per column goes with one slice of K");
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{ssq, n_partials, eps, nullptr}, nullptr, SkRope{}, stream, false};
   a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out, col_scale, act_limit, act_shift};
   a.wl = w_order;

@@ -62,8 +62,7 @@ def _declare(lib):
         "gl3_residual_inject": [P, P, P, I, I, P],
         "gl3_delta_state_floats": [I, I, I, I, I],
         "gl3_delta_prep": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, I, L, F, F, P],
-        "gl3_delta_recurrence": [P, P, P, P, P, P, I, I, I, I, I, I, L, P],
-        "gl3_delta_gated_norm": [P, P, I, I, P, I, P, I, I, I, I, F, P],
+        "gl3_delta_recurrence": [P, P, P, P, P, P, P, I, I, P, P, I, F, I, I, I, I, I, I, I, L, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
@@ -484,27 +483,23 @@ def delta_prep(proj, offsets, conv_w, A_log, dt_bias, state, cu_seqlens, seq_of_
                                     float(q_scale), _stream()), "delta_prep")
 
 
-def delta_recurrence(act, gates, state, cu_seqlens, slot_ids, out, H, G, D, Dv, taps):
-    """The rule itself, token by token for every sequence of the step from the state it holds; ``out`` [T, H Dv]
-    float32 receives the read-outs."""
-    _dev(act, "act", torch.float32); _dev(gates, "gates", torch.float32); _dev(out, "out", torch.float32)
+def delta_recurrence(act, gates, state, cu_seqlens, slot_ids, readout, proj, off_gate, norm_w, out, H, G, D, Dv, taps, eps):
+    """The rule itself, token by token for every sequence of the step from the state it holds, then the read-outs'
+    norm: ``out[t, h] = o[t, h] / rms * norm_w * silu(gate[t, h])`` (``out`` [T, H Dv] float32 or bfloat16), the gate in
+    columns ``off_gate`` .. of ``proj``; ``readout`` [T, H Dv] float32 is scratch for the raw read-outs."""
+    _dev(act, "act", torch.float32); _dev(gates, "gates", torch.float32); _dev(readout, "readout", torch.float32)
+    _dev(proj, "proj", torch.float32, contiguous=False); _dev(norm_w, "norm_w", torch.float32); _dev(out, "out")
     T = act.shape[0]
     B = _delta_common(state, cu_seqlens, slot_ids, H, G, D, Dv, taps, "delta_recurrence")
-    if act.shape != (T, 2 * G * D + H * Dv) or gates.shape != (T, 2 * H) or out.shape != (T, H * Dv):
-        raise KernelError(f"delta_recurrence: act {tuple(act.shape)}, gates {tuple(gates.shape)}, out {tuple(out.shape)}")
-    _check(library().gl3_delta_recurrence(_ptr(act), _ptr(gates), _ptr(state), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
-                                          B, H, G, D, Dv, taps, state.stride(0), _stream()), "delta_recurrence")
-
-
-def delta_gated_norm(o, proj, off_gate, weight, out, H, Dv, eps):
-    """out[t, h] = o[t, h] / rms * weight * silu(gate[t, h]), the gate in columns ``off_gate`` .. of ``proj``."""
-    _dev(o, "o", torch.float32); _dev(proj, "proj", torch.float32, contiguous=False); _dev(weight, "weight"); _dev(out, "out")
-    T = o.shape[0]
-    if (o.shape != (T, H * Dv) or out.shape != (T, H * Dv) or weight.shape != (Dv,) or proj.dim() != 2 or proj.stride(1) != 1
+    if (act.shape != (T, 2 * G * D + H * Dv) or gates.shape != (T, 2 * H) or readout.shape != (T, H * Dv)
+            or out.shape != (T, H * Dv) or norm_w.shape != (Dv,) or proj.dim() != 2 or proj.stride(1) != 1
             or proj.shape[0] != T or off_gate < 0 or off_gate + H * Dv > proj.shape[1]):
-        raise KernelError(f"delta_gated_norm: o {tuple(o.shape)}, proj {tuple(proj.shape)}, out {tuple(out.shape)}")
-    _check(library().gl3_delta_gated_norm(_ptr(o), _ptr(proj), proj.stride(0), off_gate, _ptr(weight), _code(weight, "weight"),
-                                          _ptr(out), _code(out, "out"), T, H, Dv, float(eps), _stream()), "delta_gated_norm")
+        raise KernelError(f"delta_recurrence: act {tuple(act.shape)}, gates {tuple(gates.shape)}, out {tuple(out.shape)}, "
+                          f"proj {tuple(proj.shape)}")
+    _check(library().gl3_delta_recurrence(_ptr(act), _ptr(gates), _ptr(state), _ptr(cu_seqlens), _ptr(slot_ids),
+                                          _ptr(readout), _ptr(proj), proj.stride(0), off_gate, _ptr(norm_w), _ptr(out),
+                                          _code(out, "out"), float(eps), T, B, H, G, D, Dv, taps, state.stride(0), _stream()),
+           "delta_recurrence")
 
 
 def decode_advance(token_ids, positions, kv_before, sampled, history, step):

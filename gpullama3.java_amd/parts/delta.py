@@ -103,9 +103,9 @@ class GatedDeltaRule:
                      self.dt_bias, state, ctx.cu_seqlens, ctx.seq_of_token, ctx.slot_ids, act, gates, H, G, D, Dv, taps,
                      self.spec.unit_eps, float(D) ** -0.5)
         o = ctx.buffer("delta_readout", (T, H * Dv), torch.float32)
-        K.delta_recurrence(act, gates, state, ctx.cu_seqlens, ctx.slot_ids, o, H, G, D, Dv, taps)
         y = ctx.buffer("delta_out", (T, H * Dv), self.dtype)
-        K.delta_gated_norm(o, proj, self.off_g, self.norm_w, y, H, Dv, self.spec.norm_eps)
+        K.delta_recurrence(act, gates, state, ctx.cu_seqlens, ctx.slot_ids, o, proj, self.off_g, self.norm_w, y,
+                           H, G, D, Dv, taps, self.spec.norm_eps)
         ops.linear(y, self.w_o, x, ops.EPI_ADD, ctx, col_scale=self.out_scale)
 
 

@@ -200,8 +200,7 @@ def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, gate=None, co
         for lo, hi in chunks:
             linear(a[lo:hi], w, out[lo:hi], epilogue, ctx, bias=bias, col_scale=col_scale, **(gate or {}))
         return
-    # (a bias is added once, a factor per column applied once: no slices of K with either)
-    slices = K.wide_slices(N, Kd) if bias is None and col_scale is None else 1
+    slices = K.wide_slices(N, Kd) if bias is None else 1     # (a bias is added once: no slices of K with one)
     if slices < 2:
         for lo, hi in chunks:
             K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD, bias=bias, col_scale=col_scale)
@@ -209,7 +208,7 @@ def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, gate=None, co
     settle_residual(ctx, out)
     part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
     for lo, hi in chunks:
-        K.gemm_skinny_wide(a[lo:hi], w, part[:, lo:hi], EPI_STORE)
+        K.gemm_skinny_wide(a[lo:hi], w, part[:, lo:hi], EPI_STORE, col_scale=col_scale)
     residual_written(ctx, out)
     ctx.pending = (out.data_ptr(), part)
 
@@ -243,7 +242,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
     disabled = _off(ctx if ctx is not None else getattr(a, "ctx", None))
     gate = dict(act=act, act_limit=act_limit or 0.0, act_shift=act_shift)      # the gated epilogue's rule
-    plain_sums = bias is None and col_scale is None       # (slices of K are added up later: nothing but sums may be in them)
+    plain_sums = bias is None       # (slices of K are added up later: a bias would be added once per slice; a factor per column multiplies each)
     if pack_out:
         return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias,
                                   pack_out=True, whole_lines=_whole_lines(a, w, epilogue), **gate)
@@ -280,7 +279,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
             return K.gemm_mfma(a, w, out, epilogue, bias=bias, col_scale=col_scale)
-        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or (col_scale is None and _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled)))
+        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled))
                 and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, gate, col_scale)):
             return
         rows = K.skinny_strip_rows(a.shape[0], out.shape[1], a.shape[1], epilogue)
@@ -311,7 +310,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
                 # the first slice adds into the rows, the norm that follows adds the others
                 settle_residual(ctx, out)
                 part = ctx.buffer(f"slices{slices - 1}", (slices - 1, M, out.shape[1]), torch.float32)
-                K.gemm_mfma(a, w, out, epilogue, more_slices=part, shape=shape)
+                K.gemm_mfma(a, w, out, epilogue, more_slices=part, shape=shape, col_scale=col_scale)
                 residual_written(ctx, out)
                 ctx.pending = (out.data_ptr(), part)
                 return
@@ -365,7 +364,7 @@ def _linear_wide(a, w, out, epilogue, ctx, bias=None, gate=None, col_scale=None)
             K.gemm_mfma(a, w, out, epilogue, bias=bias, col_scale=col_scale)
             return True
         return False
-    if bias is not None or col_scale is not None:     # a bias is added once, a factor per column applied once: no slices of K
+    if bias is not None:          # a bias is added once: no slices of K with one
         return False
     # into the residual stream: K in slices, added up by the norm that follows
     slices = K.wide_slices(N, Kd)
@@ -373,7 +372,7 @@ def _linear_wide(a, w, out, epilogue, ctx, bias=None, gate=None, col_scale=None)
         return False
     settle_residual(ctx, out)
     part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
-    K.gemm_skinny_wide(a, w, part, EPI_STORE)
+    K.gemm_skinny_wide(a, w, part, EPI_STORE, col_scale=col_scale)
     residual_written(ctx, out)
     ctx.pending = (out.data_ptr(), part)
     return True

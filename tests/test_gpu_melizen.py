@@ -211,7 +211,7 @@ def test_prompt_attention_on_the_matrix_cores_with_bias_and_sink(H, G, D, window
 
 # ----------------------------------------------------------------- the delta rule's kernels
 def delta_kernels(proj, shape, conv_w, A_log, dt_bias, norm_w, state, cuts, slot, eps, dtype="float32"):
-    """The three launches over one sequence cut at ``cuts``; returns the normalised, gated read-outs [T, H Dv]."""
+    """The kernels' launches over one sequence cut at ``cuts``; returns the normalised, gated read-outs [T, H Dv]."""
     from gpullama3_java_amd.csrc import lib as K
     H, G, D, Dv, taps = shape
     GD, HV = G * D, H * Dv
@@ -226,9 +226,8 @@ def delta_kernels(proj, shape, conv_w, A_log, dt_bias, norm_w, state, cuts, slot
         K.delta_prep(p, offs, dev(conv_w), dev(A_log), dev(dt_bias), state, cu, seq, slots, act, gates, H, G, D, Dv, taps,
                      1e-6, D ** -0.5)
         o = torch.empty(T, HV, device=DEV)
-        K.delta_recurrence(act, gates, state, cu, slots, o, H, G, D, Dv, taps)
         y = torch.empty(T, HV, dtype=TD[dtype], device=DEV)
-        K.delta_gated_norm(o, p, 2 * GD + HV, dev(norm_w), y, H, Dv, eps)
+        K.delta_recurrence(act, gates, state, cu, slots, o, p, 2 * GD + HV, dev(norm_w), y, H, G, D, Dv, taps, eps)
         outs.append(y.float().cpu().numpy())
         lo = hi
     return np.concatenate(outs)
