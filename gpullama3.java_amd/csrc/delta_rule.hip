@@ -31,11 +31,12 @@ struct DeltaShape {
 };
 
 // grid (T, 2 G + H + 1): a q head, a k head, a v head, or the token's decays and strengths. One wave.
+// one_each: every sequence of the step brings exactly one token (a decode step); the held inputs then move on here.
 __global__ __launch_bounds__(64) void delta_prep_kernel(
     const float* __restrict__ proj, const float* __restrict__ conv_w, const float* __restrict__ A_log,
-    const float* __restrict__ dt_bias, const float* __restrict__ state, const int* __restrict__ cu_seqlens,
+    const float* __restrict__ dt_bias, float* __restrict__ state, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_of_token, const int* __restrict__ slot_ids, float* __restrict__ act,
-    float* __restrict__ gates, DeltaShape s, float unit_eps, float q_scale) {
+    float* __restrict__ gates, DeltaShape s, float unit_eps, float q_scale, int one_each) {
   const int t = blockIdx.x, u = blockIdx.y, lane = threadIdx.x;
   const int C = 2 * s.G * s.D + s.H * s.Dv;
   const float* row = proj + (long)t * s.ldp;
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(
   }
   const int b = seq_of_token[t];
   const int first = cu_seqlens[b], i = t - first;
-  const float* held = state + (long)slot_ids[b] * s.state_stride + s.conv_off;
+  float* held = state + (long)slot_ids[b] * s.state_stride + s.conv_off;
   // the unit's channels: c0 .. c0 + n of the C convolved channels, which are columns col0 .. of the projection
   int c0, col0, n;
   if (u < s.G) { c0 = u * s.D; col0 = s.off_q + u * s.D; n = s.D; }
@@ -68,6 +69,12 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(
     y = y * dr_sigmoid(y);
     ss = fmaf(y, y, ss);
     act[(long)t * C + c] = y;
+    if (one_each && s.taps > 1) {
+      // every sequence brings one token: this lane is the only reader of the channel's held inputs, and moves them on
+      float* hc = held + (long)c * (s.taps - 1);
+      for (int jj = 0; jj + 2 < s.taps; ++jj) hc[jj] = hc[jj + 1];
+      hc[s.taps - 2] = proj[(long)t * s.ldp + col0 + e];
+    }
   }
   if (!unit) return;
   ss = wave_sum(ss);
@@ -286,12 +293,13 @@ extern "C" long gl3_delta_state_floats(int H, int G, int D, int Dv, int taps) {
 }
 
 // proj [T][ldp] float: the projection of the step's tokens. conv_w [C][taps], A_log [H], dt_bias [H] float.
-// state [slots][state_stride] float. act [T][C] and gates [T][2 H] float are written; then the held inputs move on.
+// state [slots][state_stride] float. act [T][C] and gates [T][2 H] float are written; then the held inputs move on
+// (one_each: the caller vouches that every sequence brings exactly one token, and they move on in the same launch).
 extern "C" int gl3_delta_prep(const float* proj, const float* conv_w, const float* A_log, const float* dt_bias,
                               float* state, const int* cu_seqlens, const int* seq_of_token, const int* slot_ids,
                               float* act, float* gates, int T, int B, int H, int G, int D, int Dv, int taps, int ldp,
                               int off_q, int off_k, int off_v, int off_b, int off_a, long state_stride, float unit_eps,
-                              float q_scale, hipStream_t stream) {
+                              float q_scale, int one_each, hipStream_t stream) {
   if (T == 0 || B == 0) return 0;
   GL3_REQUIRE(proj && conv_w && A_log && dt_bias && state && cu_seqlens && seq_of_token && slot_ids && act && gates &&
                   T > 0 && B > 0, "gl3_delta_prep: bad arguments");
@@ -299,9 +307,10 @@ extern "C" int gl3_delta_prep(const float* proj, const float* conv_w, const floa
   if (delta_shape(s, H, G, D, Dv, taps, ldp, off_q, off_k, off_v, off_b, off_a, state_stride)) return -1;
   GL3_REQUIRE(2 * G + H + 1 <= 65535 && B <= 65535, "gl3_delta_prep: too many heads or sequences for the grid");
   delta_prep_kernel<<<dim3(T, 2 * G + H + 1), dim3(64), 0, stream>>>(proj, conv_w, A_log, dt_bias, state, cu_seqlens,
-                                                                     seq_of_token, slot_ids, act, gates, s, unit_eps, q_scale);
+                                                                     seq_of_token, slot_ids, act, gates, s, unit_eps, q_scale, one_each);
   GL3_LAUNCH_CHECK();
-  if (taps > 1) {
+  GL3_REQUIRE(!one_each || T == B, "gl3_delta_prep: %d tokens of %d sequences are not one each", T, B);
+  if (taps > 1 && !one_each) {
     const int C = 2 * G * D + H * Dv;
     delta_conv_state_kernel<<<dim3(B, (C + 255) / 256), dim3(256), 0, stream>>>(proj, state, cu_seqlens, slot_ids, s);
     GL3_LAUNCH_CHECK();

@@ -61,7 +61,7 @@ def _declare(lib):
         "gl3_kv_write": [P, I, L, I, I, P, P, P, I, P, P, I, I, I, I, I, P],
         "gl3_residual_inject": [P, P, P, I, I, P],
         "gl3_delta_state_floats": [I, I, I, I, I],
-        "gl3_delta_prep": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, I, L, F, F, P],
+        "gl3_delta_prep": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, I, L, F, F, I, P],
         "gl3_delta_recurrence": [P, P, P, P, P, P, P, I, I, P, P, I, F, I, I, I, I, I, I, I, L, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
@@ -460,10 +460,11 @@ def _delta_common(state, cu_seqlens, slot_ids, H, G, D, Dv, taps, who):
 
 
 def delta_prep(proj, offsets, conv_w, A_log, dt_bias, state, cu_seqlens, seq_of_token, slot_ids, act, gates,
-               H, G, D, Dv, taps, unit_eps, q_scale):
+               H, G, D, Dv, taps, unit_eps, q_scale, one_token_each=False):
     """The step's q, k, v after the short convolution, silu and (q, k) the scaling to unit length into ``act``
     [T, 2 G D + H Dv], the heads' decays and write strengths into ``gates`` [T, 2 H]; then each sequence's held
-    inputs move on. ``proj`` [T, ld] float32; ``offsets``: the first columns of q, k, v, b and a in it."""
+    inputs move on. ``proj`` [T, ld] float32; ``offsets``: the first columns of q, k, v, b and a in it.
+    ``one_token_each``: the caller vouches that every sequence brings exactly one token (one launch less)."""
     _dev(proj, "proj", torch.float32, contiguous=False)
     for t, n in ((conv_w, "conv_w"), (A_log, "A_log"), (dt_bias, "dt_bias"), (act, "act"), (gates, "gates")):
         _dev(t, n, torch.float32)
@@ -480,7 +481,7 @@ def delta_prep(proj, offsets, conv_w, A_log, dt_bias, state, cu_seqlens, seq_of_
     _check(library().gl3_delta_prep(_ptr(proj), _ptr(conv_w), _ptr(A_log), _ptr(dt_bias), _ptr(state), _ptr(cu_seqlens),
                                     _ptr(seq_of_token), _ptr(slot_ids), _ptr(act), _ptr(gates), T, B, H, G, D, Dv, taps,
                                     proj.stride(0), *[int(o) for o in offsets], state.stride(0), float(unit_eps),
-                                    float(q_scale), _stream()), "delta_prep")
+                                    float(q_scale), int(bool(one_token_each) and T == B), _stream()), "delta_prep")
 
 
 def delta_recurrence(act, gates, state, cu_seqlens, slot_ids, readout, proj, off_gate, norm_w, out, H, G, D, Dv, taps, eps):

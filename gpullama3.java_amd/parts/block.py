@@ -71,9 +71,10 @@ class ParallelBlock:
 
     def forward(self, ctx, x, run, norm_after=None):
         h = PreNormBlock._whole_rows_for(self.norm, "takes_slices", ctx, x)(ctx, x)
-        if self.ffn is not None and isinstance(h, ops.Normed):
-            # a norm that a product was to take over is worked out from the rows when somebody asks for it; the
-            # feed-forward asks after the mixer has added to them, so it is worked out now
+        if self.ffn is not None and isinstance(h, ops.Normed) and not getattr(self.ffn, "folds_norm", lambda h: False)(h):
+            # a norm that a product was to take over is worked out from the rows when somebody asks for it; a
+            # feed-forward whose first product does not take it over would ask after the mixer has added to them,
+            # so it is worked out now
             h = h.materialize()
         # (both sublayers read h, and a product of the first must not prepare rows that are not whole yet)
         ctx.next_norm = None if self.ffn is not None else norm_after

@@ -101,7 +101,7 @@ class GatedDeltaRule:
         gates = ctx.buffer("delta_gates", (T, 2 * H), torch.float32)
         K.delta_prep(proj, (self.off_q, self.off_k, self.off_v, self.off_b, self.off_a), self.conv_w, self.A_log,
                      self.dt_bias, state, ctx.cu_seqlens, ctx.seq_of_token, ctx.slot_ids, act, gates, H, G, D, Dv, taps,
-                     self.spec.unit_eps, float(D) ** -0.5)
+                     self.spec.unit_eps, float(D) ** -0.5, one_token_each=bool(ctx.decode and ctx.max_q_len == 1))
         o = ctx.buffer("delta_readout", (T, H * Dv), torch.float32)
         y = ctx.buffer("delta_out", (T, H * Dv), self.dtype)
         K.delta_recurrence(act, gates, state, ctx.cu_seqlens, ctx.slot_ids, o, proj, self.off_g, self.norm_w, y,

@@ -71,6 +71,11 @@ class GatedFeedForward:
         if self.out_scale_name:
             self.out_scale = weights[self.out_scale_name].float().contiguous()
 
+    def folds_norm(self, h):
+        """Whether the first product takes over the work of the norm that ``h`` (an ``ops.Normed``) stands for."""
+        out = type("Out", (), {"dtype": self.dtype, "shape": (h.shape[0], self.F)})
+        return self.b_gate_up is None and ops.takes_folded_norm(h, self.w_gate_up, out, ops.EPI_GATED)
+
     def forward(self, ctx, h, x):
         plain = not self.limit and not self.up_shift and self.out_scale is None and self.act in K.FAST_ACTIVATIONS
         if (plain and self.b_gate_up is None and self.b_down is None

@@ -261,10 +261,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
             residual_written(ctx, out)
         return
     if isinstance(a, Normed):
-        if ("fused" not in disabled and col_scale is None and w.dtype == torch.bfloat16
-                and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
-                and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)
-                and (_whole_lines(a, w, epilogue) or K.skinny_takes(w, out.shape[0], 16))):
+        if col_scale is None and takes_folded_norm(a, w, out, epilogue):
             return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias,
                                       whole_lines=_whole_lines(a, w, epilogue), **gate)
         a = a.materialize()
@@ -321,6 +318,16 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     K.gemm_generic(a, w, out, epilogue, bias=bias, col_scale=col_scale, **gate)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
+
+
+def takes_folded_norm(a, w, out, epilogue):
+    """Whether the product of the ``Normed`` rows ``a`` with ``w`` does the norm's work itself (``out``: the product's
+    output, or anything with its ``dtype`` and ``shape``). A caller that hands one ``Normed`` to several products asks
+    before the residual rows change: what does not fold works the norm out from the rows when it runs."""
+    disabled = _off(a.ctx)
+    return ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
+            and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)
+            and (_whole_lines(a, w, epilogue) or K.skinny_takes(w, out.shape[0], 16)))
 
 
 def _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled=_NONE):
