@@ -76,11 +76,12 @@ class GQAAttention:
             self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
         self.w_q = self.w_qkv[:qn]
         without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
-        # (the strips of the copy pair up what a rotation's end pairs up; no rotation, or values of another size: a
-        # plain copy, which every product of few rows reads)
+        # (the copy as the product that rotates and writes the cache in its epilogue reads it; biased projections
+        # without a rotation, and values of another size, never take that product: a plain copy, which every product
+        # of few rows reads)
         ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
                                       bool(self.position is not None and self.position.adjacent))
-                         if self.vd == self.hs and self.position is not None else None, without=without)
+                         if self.vd == self.hs and (self.position is not None or not self.biased) else None, without=without)
         self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
         if getattr(self, "may_hold_once", False):
             # the stored order is let go where a copy in the matrix cores' order can stand for the matrix; the stored
