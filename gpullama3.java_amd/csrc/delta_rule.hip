@@ -194,33 +194,58 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
     const bool more = t0 + chunk < last;
     if (more) ask(t0 + chunk);
     const int n_here = min(chunk, last - t0);
-    for (int tt = 0; tt < n_here; ++tt) {
+    // two tokens' operands in registers in turn: the next token's reads from shared memory are on their way while
+    // the current token's chain of multiply-adds runs
+    struct Operands { float k[RPL], q[RPL], v, g, beta; };
+    auto fetch = [&](Operands& x, int tt) {
       const float* op = dr_lds + (buf * chunk + tt) * per_token;
-      const float g = op[8 * RPL + Dv], beta = op[8 * RPL + Dv + 1];
-      const float v = valid ? op[8 * RPL + j] : 0.f;
-      float kc[RPL], qc[RPL];
 #pragma unroll
       for (int ii = 0; ii < RPL; ii += 4) {
         const f4 q4 = *(const f4*)(op + r * RPL + ii), k4 = *(const f4*)(op + 4 * RPL + r * RPL + ii);
 #pragma unroll
-        for (int x = 0; x < 4; ++x) { qc[ii + x] = q4[x]; kc[ii + x] = k4[x]; }
+        for (int e = 0; e < 4; ++e) { x.q[ii + e] = q4[e]; x.k[ii + e] = k4[e]; }
       }
+      x.g = op[8 * RPL + Dv];
+      x.beta = op[8 * RPL + Dv + 1];
+      x.v = valid ? op[8 * RPL + j] : 0.f;
+    };
+    auto work = [&](const Operands& x, int tt) {
       float p4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < RPL; ++ii) {
-        S[ii] *= g;
-        p4[ii & 3] = fmaf(S[ii], kc[ii], p4[ii & 3]);
+        S[ii] *= x.g;
+        p4[ii & 3] = fmaf(S[ii], x.k[ii], p4[ii & 3]);
       }
       const float part = dr_sum4((p4[0] + p4[1]) + (p4[2] + p4[3]));
-      const float uu = beta * (v - part);
+      const float uu = x.beta * (x.v - part);
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < RPL; ++ii) {
-        S[ii] = fmaf(kc[ii], uu, S[ii]);
-        o4[ii & 3] = fmaf(S[ii], qc[ii], o4[ii & 3]);
+        S[ii] = fmaf(x.k[ii], uu, S[ii]);
+        o4[ii & 3] = fmaf(S[ii], x.q[ii], o4[ii & 3]);
       }
       const float read = dr_sum4((o4[0] + o4[1]) + (o4[2] + o4[3]));
       if (r == 0 && valid) o[(long)(t0 + tt) * H * Dv + (long)h * Dv + j] = read;
+    };
+    if constexpr (RPL <= 24 && MAXT <= 512) {
+      // (pairs of tokens without a branch between them, so that the end of one token's work, which nothing waits
+      // for, can be scheduled into the start of the next one's)
+      Operands xa, xb;
+      fetch(xa, 0);
+      int tt = 0;
+      for (; tt + 2 <= n_here; tt += 2) {
+        fetch(xb, tt + 1);
+        work(xa, tt);
+        fetch(xa, min(tt + 2, n_here - 1));
+        work(xb, tt + 1);
+      }
+      if (tt < n_here) work(xa, tt);
+    } else {                              // (long keys, or a block of sixteen waves: two tokens' operands beside the matrix do not fit the registers)
+      Operands xa;
+      for (int tt = 0; tt < n_here; ++tt) {
+        fetch(xa, tt);
+        work(xa, tt);
+      }
     }
     if (more) put(buf ^ 1);
     __syncthreads();
