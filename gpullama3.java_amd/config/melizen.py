@@ -219,7 +219,11 @@ class MelizenConfiguration:
             run_order=self.run_order(),
             final_norm=NormSpec(dim=d, eps=eps, names={"weight": "final.norm"}, weight_offset=1.0),
             max_positions=self.max_positions, tie_embeddings=False, embedding_name="embed", head_name="head",
-            stop_ids=self.stop_ids, position_table_name="pos")
+            stop_ids=self.stop_ids, position_table_name="pos",
+            # (a folder may hold the scale of a feed-forward that a layer does not have, and the passes' vectors of a
+            # loop over no layer: nothing reads them)
+            unused_tensor_names=tuple(f"l{i}.ls2" for i, lay in enumerate(self.layers) if lay.mlp is None)
+            + (() if self.looped else ("loop.step",)))
 
 
 register_architecture("Melizen", MelizenConfiguration)

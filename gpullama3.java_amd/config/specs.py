@@ -162,3 +162,4 @@ class ModelSpec:
     logit_scale: Optional[float] = None           # the logits times this
     head_bias_name: Optional[str] = None          # a stored [vocab] vector added to the logits (before the scale)
     logit_softcap: Optional[float] = None         # the logits become cap * tanh(logits / cap) (after the scale)
+    unused_tensor_names: tuple = ()               # stored names that a folder may hold although nothing reads them

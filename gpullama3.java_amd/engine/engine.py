@@ -134,7 +134,8 @@ class Engine:
         config = load_config(folder)
         probe = DecoderModel(config.model_spec(), _dtype(dtype), "cpu")
         check_layout(probe.cache_needs()[0], kw.get("page_size", 64))       # before the weights are read
-        weights = load_weights(folder, probe.expected(), _dtype(dtype), dev)
+        weights = load_weights(folder, probe.expected(), _dtype(dtype), dev,
+                               ignore=getattr(probe.spec, "unused_tensor_names", ()))
         return cls(config, weights, dtype=dtype, device=device, **kw)
 
     @classmethod

@@ -35,6 +35,12 @@ class GQAAttention:
         if self.H % self.Kh:
             raise ValueError(f"{self.H} heads are not a multiple of {self.Kh} kv heads")
         self.vd = spec.v_head_dim if getattr(spec, "v_head_dim", None) else self.hs
+        # The cache keeps heads in tiles of 16 elements. Without a rotation a head of any other size is stored with
+        # zero rows (q, k, v) and zero columns (o) up to the next multiple of 16: scores and outputs are the same
+        # numbers, and every kernel sees the padded sizes.
+        self.hs_stored, self.vd_stored = self.hs, self.vd
+        if spec.position is None:
+            self.hs, self.vd = -(-self.hs // 16) * 16, -(-self.vd // 16) * 16
         self.window = spec.window
         self.sink = getattr(spec, "sink", None)
         bias = getattr(spec, "distance_bias", None)
@@ -52,7 +58,7 @@ class GQAAttention:
         self.w_qkv = self.w_q = self.w_o = self.b_qkv = self.b_o = None
 
     def tensors(self):
-        n, d, hs, vd = self.names, self.d, self.hs, self.vd
+        n, d, hs, vd = self.names, self.d, self.hs_stored, self.vd_stored
         out = {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
                n["v"]: TensorSpec((self.Kh * vd, d)), n["o"]: TensorSpec((d, self.H * vd))}
         if self.biased:
@@ -67,6 +73,8 @@ class GQAAttention:
 
     def load(self, weights):
         n = self.names
+        if (self.hs, self.vd) != (self.hs_stored, self.vd_stored):
+            weights = _PaddedHeads(weights, self)
         parts = [weights[n["q"]], weights[n["k"]], weights[n["v"]]]
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         self.w_qkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
@@ -134,6 +142,34 @@ class GQAAttention:
         K.kv_write(qkv, qn, qn + kn, ctx.positions, ops._table_rows(ctx), table, k_cache, v_cache, self.Kh, self.hs,
                    self.vd, k_cache.shape[2])
         return qkv
+
+
+class _PaddedHeads:
+    """The weights of an attention whose heads are stored in other sizes than the cache's tiles take, as the part
+    reads them: every head of q, k (rows), v (rows), their biases and o (columns) padded with zeros. What the part
+    writes back (the stacked rows under the stored names) goes to the model's weights as it is: padded."""
+
+    def __init__(self, weights, part):
+        self.weights, self.part = weights, part
+
+    def __getitem__(self, name):
+        p, n, w = self.part, self.part.names, self.weights[name]
+        heads = {n["q"]: (p.H, p.hs_stored, p.hs), n["k"]: (p.Kh, p.hs_stored, p.hs), n["v"]: (p.Kh, p.vd_stored, p.vd),
+                 n.get("q_bias"): (p.H, p.hs_stored, p.hs), n.get("k_bias"): (p.Kh, p.hs_stored, p.hs),
+                 n.get("v_bias"): (p.Kh, p.vd_stored, p.vd)}
+        if name in heads and w.shape[0] == heads[name][0] * heads[name][1]:
+            H, d_in, d_out = heads[name]
+            out = torch.zeros((H, d_out) + tuple(w.shape[1:]), dtype=w.dtype, device=w.device)
+            out[:, :d_in] = w.reshape((H, d_in) + tuple(w.shape[1:]))
+            return out.reshape((H * d_out,) + tuple(w.shape[1:])).contiguous()
+        if name == n["o"] and w.shape[1] == p.H * p.vd_stored:
+            out = torch.zeros((w.shape[0], p.H, p.vd), dtype=w.dtype, device=w.device)
+            out[:, :, :p.vd_stored] = w.reshape(w.shape[0], p.H, p.vd_stored)
+            return out.reshape(w.shape[0], p.H * p.vd).contiguous()
+        return w
+
+    def __setitem__(self, name, value):
+        self.weights[name] = value
 
 
 register_part("mixer", "attention", GQAAttention)

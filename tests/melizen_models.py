@@ -46,7 +46,8 @@ STRAIGHT = {
 # the loop in the middle and at the end of the list
 LOOP_AT_END = {
     "architecture": "Melizen", "vocab": 128, "width": 64, "max_positions": 320, "norm": {"eps": 1e-5},
-    "layers": [_attn(2, 1, 16, 32, 9, 0.3, _mlp(96, 2.0)), _delta(2, 1, 16, 16, 4, _mlp(96, 2.0)),
+    # (the first attention's heads are no multiples of the cache's tiles: they are padded when the weights load)
+    "layers": [_attn(2, 1, 24, 40, 9, 0.3, _mlp(96, 2.0)), _delta(2, 1, 16, 16, 4, _mlp(96, 2.0)),
                _attn(4, 2, 32, 16, 33, 0.2, None)],
     "loop": {"start": 1, "stop": 3, "times": 2},
 }

@@ -481,3 +481,27 @@ def test_the_command_line_takes_the_model(tmp_path, capsys):
         assert t == int(np.argmax(P.forward(cfg, W, seq)[-1]))
         seq.append(t)
     assert len(got) >= 3
+
+
+def test_a_folder_may_hold_tensors_that_nothing_reads(tmp_path):
+    """The scale of a feed-forward that a layer does not have is tolerated; any other unknown tensor is reported."""
+    import json
+    import os
+    from safetensors.torch import save_file
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.weights import WeightsError
+    folder, cfg, W = model("looped")                    # its layer 2 has no feed-forward
+    for extra, ok in (("l2.ls2", True), ("l2.ls3", False)):
+        d = tmp_path / extra
+        os.makedirs(d)
+        tensors = {k: torch.tensor(v).to(torch.bfloat16) for k, v in W.items()}
+        tensors[extra] = torch.ones(cfg["width"], dtype=torch.bfloat16)
+        save_file(tensors, str(d / "model.safetensors"))
+        (d / "config.json").write_text(json.dumps(cfg))
+        if ok:
+            eng = Engine.from_folder(str(d), dtype="float32", max_tokens=256, n_slots=2)
+            toks = tokens("looped", 40, 12)
+            close(eng.step([(eng.take_slot(), toks)], want="all").cpu().numpy(), P.forward(cfg, W, toks), "float32")
+        else:
+            with pytest.raises(WeightsError, match="l2.ls3"):
+                Engine.from_folder(str(d), dtype="float32", max_tokens=256, n_slots=2)
