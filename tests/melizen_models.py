@@ -51,11 +51,11 @@ LOOP_AT_END = {
                _attn(4, 2, 32, 16, 33, 0.2, None)],
     "loop": {"start": 1, "stop": 3, "times": 2},
 }
-# head sizes that the matrix-core attention kernels are built for (values of the keys' size), one kv head for eight
-# query heads, widths in whole tiles: what a bfloat16 engine runs on its fast paths
+# head sizes that the matrix-core attention kernels are built for (values of the keys' size), two kv heads for
+# eight query heads, widths in whole tiles: what a bfloat16 engine runs on its fast paths
 TILED = {
-    "architecture": "Melizen", "vocab": 512, "width": 128, "max_positions": 512, "norm": {"eps": 1e-5},
-    "layers": [_attn(8, 1, 64, 64, 100, 0.125, _mlp(256, 2.0)), _delta(4, 2, 64, 64, 4, _mlp(256, 2.0)),
+    "architecture": "Melizen", "vocab": 640, "width": 128, "max_positions": 512, "norm": {"eps": 1e-5},
+    "layers": [_attn(8, 2, 64, 64, 100, 0.125, _mlp(256, 4.0)), _delta(4, 2, 64, 64, 3, _mlp(256, 1.5)),
                _attn(4, 4, 32, 32, None, 0.18, _mlp(128, 1.0)), _attn(2, 1, 96, 96, 70, 0.1, None),
                _attn(2, 2, 128, 128, 130, 0.09, _mlp(128, 3.0))],
     "loop": {"start": 1, "stop": 2, "times": 2},
