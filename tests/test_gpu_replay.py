@@ -99,6 +99,8 @@ def test_replay_refuses_more_than_the_cache_holds(tmp_path):
     folder, _, _ = model("A")
     rp = Replay(folder, "float32", tmp_path, max_tokens=64)
     rp.step([("a", [1] * 60, [59])])
-    rp.p.stdin.write(json.dumps({"step": 1, "entries": [{"id": "b", "tokens": [1], "want": [0]}], "end": []}) + "\n")
+    # (the runner keeps a page to spare for each of up to 64 requests whose last page is partly filled)
+    more = [{"id": f"b{i}", "tokens": [1], "want": [0]} for i in range(70)]
+    rp.p.stdin.write(json.dumps({"step": 1, "entries": more, "end": []}) + "\n")
     rp.p.stdin.close()
-    assert rp.p.wait(timeout=60) != 0                           # a second request needs a second page
+    assert rp.p.wait(timeout=60) != 0                           # seventy more requests need seventy more pages
