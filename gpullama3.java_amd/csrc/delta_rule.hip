@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(const float* __re
   }
 }
 
-// The rule itself and the read-out's norm. grid (H, B), a block of ceil(Dv / 16) waves: wave w owns the 16 value
+// The rule itself and the read-out's norm. grid (H, B, blocks a head: 1 unless the launcher deals a prompt's head out), a block of ceil(Dv / 16) waves: wave w owns the 16 value
 // columns 16 w .. of head h's matrix, lane (r, c) of it the rows r, r + 4, ... of column c (RPL rows a lane), so a
 // token costs a lane RPL multiply-adds for each of S^T k, the update and S^T q, and the sums over the four lanes of
 // a column are two lane swaps each (no trip through shared memory). The tokens' operands (k, q, v, decay,
@@ -118,36 +118,49 @@ __device__ __forceinline__ float dr_sum4(float p) {   // the sum over lanes l, l
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <int RPL, typename TO, int MAXT>
+// RG: the lanes a column's rows are dealt out to, 4 (16 columns a wave) or 8 (8 columns a wave: twice the waves with
+// half the work per token each, which is what a prompt's long chains of tokens want; the state lies the same).
+template <int RG>
+__device__ __forceinline__ float dr_sum_rows(float p) {
+  if (RG == 8)    // lane l ^ 8 is 8 places round the row of 16
+    p += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(p), 0x128, 0xf, 0xf, false));
+  return dr_sum4(p);
+}
+
+template <int RPL, typename TO, int MAXT, int RG>
 __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
     const float* __restrict__ act, const float* __restrict__ gates, float* __restrict__ state,
     const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids, float* __restrict__ o,
     const float* __restrict__ proj, int ldp, int off_gate, const float* __restrict__ norm_w, TO* __restrict__ y,
-    float eps, DeltaShape s, int chunk, int norm_here) {
+    float eps, DeltaShape s, int chunk, int norm_here, int own_waves) {
   extern __shared__ __attribute__((aligned(16))) float dr_lds[];   // two buffers of chunk * per_token floats
   typedef float f4 __attribute__((ext_vector_type(4)));
   const int h = blockIdx.x, b = blockIdx.y;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane >> 4, c = lane & 15;
+  constexpr int COLS = 64 / RG;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane / COLS, c = lane % COLS;
   const int D = s.D, H = s.H, Dv = s.Dv;
-  const int j = wave * 16 + c;
-  const bool valid = j < Dv;
+  // (a head's columns may be dealt out to several blocks, blockIdx.z: own_waves waves of columns each)
+  const int j = ((int)blockIdx.z * own_waves + wave) * COLS + c;
+  const bool valid = wave < own_waves && j < Dv;
   const int C = 2 * s.G * D + H * Dv;
   const int kvh = h / (H / s.G);
   const int first = cu_seqlens[b], last = cu_seqlens[b + 1];
   if (last <= first) return;
   const int CT = (Dv + 15) / 16;
-  const bool owner = wave < CT;       // (a block may have more waves than tiles of columns: they only help to load)
-  float* tile = state + (long)slot_ids[b] * s.state_stride + ((long)(h * CT + (owner ? wave : 0)) * D) * 16;
+  const bool owner = wave < own_waves && j < CT * 16;     // (a block may have more waves than columns to own: they only help to load)
+  // the lane's column in the state's tiles of 16 columns: row i of it at [16 i]
+  float* tile = state + (long)slot_ids[b] * s.state_stride + ((long)(h * CT + (owner ? j / 16 : 0)) * D) * 16 + (j & 15);
   float S[RPL];
 #pragma unroll
   for (int ii = 0; ii < RPL; ++ii) {
-    const int i = r + 4 * ii;
-    S[ii] = (owner && i < D) ? tile[(long)i * 16 + c] : 0.f;
+    const int i = r + RG * ii;
+    S[ii] = (owner && i < D) ? tile[(long)i * 16] : 0.f;
   }
   // A token's operands in a chunk's buffer: q | k | v [Dv] | decay, strength, where q and k lie as the lanes read
-  // them: row r + 4 ii at [r][ii], RPL places a lane (rows beyond D stay zero), so a lane's share is 16-byte reads.
+  // them: row r + RG ii at [r][ii], RPL places a lane (rows beyond D stay zero), so a lane's share is 16-byte reads.
   const int per_src = 2 * D + Dv + 2;                           // what a token brings
-  const int per_token = 8 * RPL + ((Dv + 2 + 3) & ~3);          // what it takes in the buffer
+  constexpr int VEC = RG * RPL;                                 // places of q, and of k
+  const int per_token = 2 * VEC + ((Dv + 2 + 3) & ~3);          // what it takes in the buffer
   const int n_src = chunk * per_src;
   const long q_at = (long)kvh * D, k_at = (long)s.G * D + (long)kvh * D, v_at = 2L * s.G * D + (long)h * Dv;
   const int threads = blockDim.x;
@@ -178,9 +191,9 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
         int at;
         if (f < 2 * D) {
           const int which = f >= D, i = f - which * D;
-          at = which * 4 * RPL + (i & 3) * RPL + (i >> 2);
+          at = which * VEC + (i % RG) * RPL + i / RG;
         } else {
-          at = 8 * RPL + (f - 2 * D);
+          at = 2 * VEC + (f - 2 * D);
         }
         dr_lds[(buf * chunk + tt) * per_token + at] = held[n];
       }
@@ -201,13 +214,13 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
       const float* op = dr_lds + (buf * chunk + tt) * per_token;
 #pragma unroll
       for (int ii = 0; ii < RPL; ii += 4) {
-        const f4 q4 = *(const f4*)(op + r * RPL + ii), k4 = *(const f4*)(op + 4 * RPL + r * RPL + ii);
+        const f4 q4 = *(const f4*)(op + r * RPL + ii), k4 = *(const f4*)(op + VEC + r * RPL + ii);
 #pragma unroll
         for (int e = 0; e < 4; ++e) { x.q[ii + e] = q4[e]; x.k[ii + e] = k4[e]; }
       }
-      x.g = op[8 * RPL + Dv];
-      x.beta = op[8 * RPL + Dv + 1];
-      x.v = valid ? op[8 * RPL + j] : 0.f;
+      x.g = op[2 * VEC + Dv];
+      x.beta = op[2 * VEC + Dv + 1];
+      x.v = valid ? op[2 * VEC + j] : 0.f;
     };
     auto work = [&](const Operands& x, int tt) {
       float p4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -216,7 +229,7 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
         S[ii] *= x.g;
         p4[ii & 3] = fmaf(S[ii], x.k[ii], p4[ii & 3]);
       }
-      const float part = dr_sum4((p4[0] + p4[1]) + (p4[2] + p4[3]));
+      const float part = dr_sum_rows<RG>((p4[0] + p4[1]) + (p4[2] + p4[3]));
       const float uu = x.beta * (x.v - part);
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -224,7 +237,7 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
         S[ii] = fmaf(x.k[ii], uu, S[ii]);
         o4[ii & 3] = fmaf(S[ii], x.q[ii], o4[ii & 3]);
       }
-      const float read = dr_sum4((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      const float read = dr_sum_rows<RG>((o4[0] + o4[1]) + (o4[2] + o4[3]));
       if (r == 0 && valid) o[(long)(t0 + tt) * H * Dv + (long)h * Dv + j] = read;
     };
     if constexpr (RPL <= 24 && MAXT <= 512) {
@@ -253,8 +266,8 @@ __global__ __launch_bounds__(MAXT) void delta_recurrence_kernel(
   }
 #pragma unroll
   for (int ii = 0; ii < RPL; ++ii) {
-    const int i = r + 4 * ii;
-    if (owner && i < D) tile[(long)i * 16 + c] = S[ii];
+    const int i = r + RG * ii;
+    if (owner && i < D) tile[(long)i * 16] = S[ii];
   }
   // (steps of many tokens a sequence: a launch of its own, with a wave to every token and head, normalises them)
   if (!norm_here) return;
@@ -360,8 +373,20 @@ extern "C" int gl3_delta_recurrence(const float* act, const float* gates, float*
   GL3_REQUIRE(off_gate >= 0 && off_gate + H * Dv <= ldp, "gl3_delta_recurrence: the gate's columns %d .. of rows of %d", off_gate, ldp);
   GL3_REQUIRE(y_dtype == GL3_F32 || y_dtype == GL3_BF16, "gl3_delta_recurrence: unknown dtype %d", y_dtype);
   // as many waves as the columns need, and as the loads of a chunk of operands need (DR_NLD a thread)
+  // the read-outs' norm: by the block that made them where a sequence brings few tokens (a decode step), else by a
+  // launch of its own with a wave to every token and head (a block's few waves would walk a prompt's tokens one by one)
+  const int norm_here = T <= 4 * B;
+  // a column's rows over 8 lanes for prompts (long chains of tokens: half the work per token and wave) where that
+  // makes at most eight waves, over 4 else (values of 128: sixteen waves of 8 columns were 5% slower than eight of 16)
+  const int rg = (!norm_here && D >= 32 && Dv <= 64) ? 8 : 4;
+  const int cols = 64 / rg;
   // (fewer tokens a chunk where that keeps the block at the waves its columns need, or at four)
-  const int col_waves = (Dv + 15) / 16;
+  // (A head's columns could be dealt out to several blocks, grid z; with blocks of four waves of 8 columns a prompt of
+  // 2,048 tokens was slower than with one block of eight, 12.8 against 12.1 ms for sixteen layers: every block stages
+  // all of a token's operands, in shorter chunks. One block a head.)
+  const int all_col_waves = (Dv + cols - 1) / cols;
+  const int col_waves = all_col_waves;
+  const int split = 1;
   int chunk = DR_CHUNK, waves = col_waves;
   for (;; chunk /= 2) {
     waves = col_waves;
@@ -369,17 +394,21 @@ extern "C" int gl3_delta_recurrence(const float* act, const float* gates, float*
     if (waves <= (col_waves > 4 ? col_waves : 4) || chunk == 1) break;
   }
   GL3_REQUIRE(waves <= 16, "gl3_delta_recurrence: keys of %d with values of %d need more than a block's threads", D, Dv);
-  dim3 grid(H, B), block(waves * 64);
-  // the read-outs' norm: by the block that made them where a sequence brings few tokens (a decode step), else by a
-  // launch of its own with a wave to every token and head (a block's few waves would walk a prompt's tokens one by one)
-  const int norm_here = T <= 4 * B;
-  const int rows = (D + 3) / 4;
+  dim3 grid(H, B, split), block(waves * 64);
+  const int rows = (D + rg - 1) / rg;
   const int rpl = rows <= 4 ? 4 : rows <= 8 ? 8 : rows <= 16 ? 16 : rows <= 24 ? 24 : rows <= 32 ? 32 : rows <= 48 ? 48 : 64;
-  const size_t lds = 2 * (size_t)chunk * (8 * rpl + ((Dv + 2 + 3) & ~3)) * sizeof(float);
+  const size_t lds = 2 * (size_t)chunk * (2 * rg * rpl + ((Dv + 2 + 3) & ~3)) * sizeof(float);
   GL3_REQUIRE(lds <= 64 * 1024, "gl3_delta_recurrence: a chunk's operands of %zu bytes exceed shared memory", lds);
-#define GO3(R, TO, MAXT)                                                                                                \
-  delta_recurrence_kernel<R, TO, MAXT><<<grid, block, lds, stream>>>(act, gates, state, cu_seqlens, slot_ids, o, proj, ldp, \
-                                                                     off_gate, norm_w, (TO*)y, eps, s, chunk, norm_here)
+#define GO4(R, TO, MAXT, RGV)                                                                                                  \
+  delta_recurrence_kernel<R, TO, MAXT, RGV><<<grid, block, lds, stream>>>(act, gates, state, cu_seqlens, slot_ids, o, proj, ldp, \
+                                                                          off_gate, norm_w, (TO*)y, eps, s, chunk, norm_here, col_waves)
+#define GO3(R, TO, MAXT)                                                       \
+  do {                                                                         \
+    if constexpr (R <= 32) {                                                   \
+      if (rg == 8) { GO4(R, TO, MAXT, 8); break; }                             \
+    }                                                                          \
+    GO4(R, TO, MAXT, 4);                                                       \
+  } while (0)
 #define GO2(R, TO)                                                             \
   do {                                                                         \
     if (waves <= 4) GO3(R, TO, 256);                                           \
@@ -403,6 +432,7 @@ extern "C" int gl3_delta_recurrence(const float* act, const float* gates, float*
 #undef GO
 #undef GO2
 #undef GO3
+#undef GO4
   GL3_LAUNCH_CHECK();
   if (!norm_here) {
     GL3_REQUIRE(T <= 2147483647 / 64, "gl3_delta_recurrence: %d tokens exceed the grid", T);
