@@ -42,6 +42,7 @@ class KVNeed:
     dtype: Optional[torch.dtype] = None      # None: the engine's; a mixer whose kernels keep something else says so
     v_head_dim: Optional[int] = None         # None: as the keys'
     values: bool = True                      # False: no second array (``layer_kv`` then gives (keys, None))
+    keep_first: int = 0                      # with a window: the sequence's first positions that stay visible (and stored)
 
     @property
     def value_dim(self):
@@ -201,7 +202,9 @@ class Cache:
                 continue
             pages = self.slots.pages[s][g]
             first_seen = max(0, self.slots.length[s] + 1 - window) // self.page_size
-            gone = [i for i in range(min(first_seen, len(pages))) if pages[i]]
+            # (the pages of the first positions that every later token still sees are held to the sequence's end)
+            kept = -(-int(getattr(group.need, "keep_first", 0) or 0) // self.page_size)
+            gone = [i for i in range(kept, min(first_seen, len(pages))) if pages[i]]
             if gone:
                 group.pool.give_back([pages[i] for i in gone])
                 for i in gone:

@@ -48,11 +48,33 @@ def load_config(folder):
     with open(path) as f:
         d = json.load(f)
     cfg = config_from_dict(d)
+    if hasattr(cfg, "with_tensor_shapes"):
+        # an architecture some of whose sizes only the weights give reads them from the files' headers
+        cfg = cfg.with_tensor_shapes(_stored_shapes(folder))
     gen = os.path.join(folder, "generation_config.json")
     if os.path.isfile(gen) and not cfg.stop_ids:
         with open(gen) as f:
             cfg = cfg.with_stop_ids(_as_ids(json.load(f).get("eos_token_id")))
     return cfg
+
+
+def _stored_shapes(folder):
+    """Stored name -> shape of every tensor in the folder's safetensors files (headers only); {} without files."""
+    from ..weights.loader import weight_files
+    from ..weights.safetensors_io import SafetensorsFile
+    out = {}
+    try:
+        paths = weight_files(folder)
+    except FileNotFoundError:
+        return out
+    for p in paths:
+        f = SafetensorsFile(p)
+        try:
+            for name in f.names():
+                out[name] = tuple(f.shape(name))
+        finally:
+            f.close()
+    return out
 
 
 def _as_ids(v):

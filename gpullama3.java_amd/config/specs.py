@@ -23,12 +23,18 @@ class Llama3RopeScaling:
 
 
 @dataclass(frozen=True)
+class LinearRopeScaling:
+    """Every frequency divided by ``factor`` (positions read as ``factor`` times closer together)."""
+    factor: float
+
+
+@dataclass(frozen=True)
 class RotarySpec:
     """Rotary position encoding of queries and keys."""
     kind: str = "rotary"
     head_dim: int = 0
     theta: float = 10000.0
-    scaling: Optional[Llama3RopeScaling] = None
+    scaling: object = None       # None, a Llama3RopeScaling or a LinearRopeScaling
     pairing: str = "half"        # "half": (j, j + hs/2); "adjacent": (2j, 2j+1)
     max_positions: int = 0
 
@@ -72,6 +78,53 @@ class AttentionSpec:
     sink: Optional[float] = None      # the score of a key without a value that every query sees (it takes its share
                                       # of the softmax's weights and adds nothing); None: no such key
     out_scale_name: Optional[str] = None   # a stored [hidden] vector that the mixer's output is multiplied by
+    keep_first: int = 0               # with a window: the first n positions of a sequence stay visible to every later query
+    value_position: Optional[RotarySpec] = None   # values are rotated by their own position before they are cached (over the
+                                      # whole value head), and each head's output is turned back by the query's position
+    out_mult: float = 1.0             # a constant that the mixer's output is multiplied by
+    # (a name ``head_gate`` among ``names``: a stored [n_heads, hidden] matrix; head h's output is multiplied by
+    # sigmoid of its row's product with the mixer's input, before the output projection)
+
+
+@dataclass(frozen=True)
+class MinGRUSpec:
+    """A gated recurrence per channel whose gates read the current token alone (``parts/mingru.py``):
+    ``S <- (1 - z) S + z c`` with z = sigmoid(W_z h + b_z), c = g(W_x h + b_x), g(u) = u + 1/2 for u >= 0 and
+    sigmoid(u) below; the output projection reads ``S * silu(W_g h)``."""
+    kind: str = "mingru"
+    hidden: int = 0
+    width: int = 0
+    names: dict = field(default_factory=dict)
+    out_mult: float = 1.0
+
+
+@dataclass(frozen=True)
+class TimeMixSpec:
+    """A matrix per head [head_dim, head_dim] in 32-bit that every token decays per key channel and adds its
+    key-value product to; the read-out sees the current token's product times a learned bonus per channel
+    (``parts/time_mix.py``). Every projection reads its own blend of the token's input and the previous token's."""
+    kind: str = "time_mix"
+    hidden: int = 0
+    n_heads: int = 0
+    head_dim: int = 0
+    decay_rank: int = 0               # the inner size of the decay's two-step projection
+    norm_eps: float = 1e-5            # the read-out's norm per head
+    names: dict = field(default_factory=dict)
+    out_mult: float = 1.0
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Two mixers that read the same input; each one's output is normalised over the model width with a weight of its
+    own, and ``weight`` times their sum is the mixer's output (``parts/side_by_side.py``)."""
+    kind: str = "side_by_side"
+    hidden: int = 0
+    left: object = None
+    right: object = None
+    norm_eps: float = 1e-5
+    weight: float = 0.5
+    names: dict = field(default_factory=dict)     # "left_norm", "right_norm": the stored [hidden] weights
+    out_mult: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -105,6 +158,7 @@ class GatedFeedForwardSpec:
     limit: Optional[float] = None
     up_shift: float = 0.0
     out_scale_name: Optional[str] = None   # a stored [hidden] vector that the output is multiplied by
+    out_mult: float = 1.0                  # a constant that the output is multiplied by
 
 
 @dataclass(frozen=True)
@@ -129,7 +183,7 @@ class Run:
     """
     layer: int
     reads: Optional[int] = None
-    before: Optional["Inject"] = None     # what is added to the residual rows right before this entry runs
+    before: object = None                 # an Inject or a Remix: what happens to the residual rows right before this entry runs
 
 
 @dataclass(frozen=True)
@@ -140,6 +194,24 @@ class Inject:
     vector_name: Optional[str] = None
     vector_rows: int = 0
     row: int = 0
+
+
+@dataclass(frozen=True)
+class Remix:
+    """The residual rows are replaced by a learned mixture of themselves and the embedding's output:
+    ``x <- W [x; x0]`` with the stored matrix ``weight_name`` ([hidden, 2 hidden], the columns for x first)."""
+    weight_name: str = ""
+
+
+@dataclass(frozen=True)
+class PairEmbedding:
+    """A second embedding row per token, looked up by a hash of (previous token, token):
+    row ``(previous * mul_prev + token * mul_cur) mod buckets`` of the stored table ``table_name``
+    ([buckets + 1, hidden]); a sequence's first token takes the last row. The previous token is kept per sequence."""
+    table_name: str = ""
+    buckets: int = 0
+    mul_prev: int = 0
+    mul_cur: int = 0
 
 
 @dataclass(frozen=True)
@@ -163,3 +235,4 @@ class ModelSpec:
     head_bias_name: Optional[str] = None          # a stored [vocab] vector added to the logits (before the scale)
     logit_softcap: Optional[float] = None         # the logits become cap * tanh(logits / cap) (after the scale)
     unused_tensor_names: tuple = ()               # stored names that a folder may hold although nothing reads them
+    pair_embedding: Optional[PairEmbedding] = None   # a row per (previous token, token) added to the embedding's output

@@ -15,7 +15,8 @@
 // (v_head_dim); a bias that grows with the distance, score - slopes[h] * (p - key), one slope per
 // query head; and a sink, a key that every query sees with the score `sink` and whose value is
 // zero, so that the weights of the real keys sum to less than one: exp(s_j) / (exp(sink) + sum exp(s)).
-// The sink is the running softmax's starting point (maximum = sink, sum = 1).
+// The sink is the running softmax's starting point (maximum = sink, sum = 1). And a window that keeps a sequence's
+// first keys visible (keep_first): query p sees key j <= p if p - j < window or j < keep_first.
 #include "common.h"
 
 #define ATT_MAX_HS 256
@@ -25,7 +26,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, T* __restrict__ out, long out_stride, int n_heads, int n_kv, int head_dim, int v_head_dim,
-    int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink) {
+    int page_size, int window, float scale, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
   __shared__ float qs[ATT_MAX_HS];
   __shared__ float ps[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -39,9 +40,14 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   const float slope = slopes ? slopes[h] : 0.f;
   float m = has_sink ? sink : -INFINITY, l = has_sink ? 1.f : 0.f;
   float acc[ATT_MAX_HS / 64] = {};
-  for (int base = lo; base <= p; base += 64) {
+  // with a window, the sequence's first keep_first keys stay visible: those of them that lie before the window are
+  // visited first, in chunks of their own, then the window's keys
+  const int kept = keep_first < lo ? keep_first : lo;
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+  const int from = run == 0 ? 0 : lo, to = run == 0 ? kept - 1 : p;
+  for (int base = from; base <= to; base += 64) {
     const int key = base + lane;
-    const bool valid = key <= p;
+    const bool valid = key <= to;
     float s = -INFINITY;
     if (valid) {
       const T* kp = k_cache + ((long)bt[key / page_size] * n_kv + c) * page_size * head_dim;
@@ -57,7 +63,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     __syncthreads();
     ps[lane] = pe;
     __syncthreads();
-    const int n_valid = (p - base + 1 < 64) ? p - base + 1 : 64;
+    const int n_valid = (to - base + 1 < 64) ? to - base + 1 : 64;
 #pragma unroll
     for (int r = 0; r < ATT_MAX_HS / 64; ++r) acc[r] *= alpha;
     for (int j = 0; j < n_valid; ++j) {
@@ -74,6 +80,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     }
     m = m_new;
   }
+  }
   T* op = out + (long)t * out_stride + (long)h * v_head_dim;
 #pragma unroll
   for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
@@ -86,7 +93,7 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
                                      const int* positions, const int* seq_of_token, const int* block_table,
                                      int table_stride, void* out, long out_stride, int n_tokens, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int v_head_dim,
-                                     const float* slopes, int has_sink, float sink, hipStream_t stream) {
+                                     const float* slopes, int has_sink, float sink, int keep_first, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
               "gl3_attention_generic: null argument");
@@ -98,6 +105,7 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
               "gl3_attention_generic: v_head_dim %d is not a multiple of 16 up to %d", v_head_dim, ATT_MAX_HS);
   GL3_REQUIRE(n_heads <= 65535, "gl3_attention_generic: %d heads exceed the grid", n_heads);
   GL3_REQUIRE(page_size > 0 && table_stride > 0, "gl3_attention_generic: bad paging");
+  GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_generic: %d kept first keys without a window", keep_first);
   GL3_REQUIRE(page_size % 32 == 0 && head_dim % 16 == 0,
               "gl3_attention_generic: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16", page_size,
               head_dim);
@@ -106,12 +114,12 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
     attention_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, positions, seq_of_token, block_table,
         table_stride, (float*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale, slopes, has_sink,
-        sink);
+        sink, keep_first);
   else if (dtype == GL3_BF16)
     attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,
         block_table, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, head_dim, v_head_dim, page_size, window, scale,
-        slopes, has_sink, sink);
+        slopes, has_sink, sink, keep_first);
   else GL3_REQUIRE(false, "gl3_attention_generic: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;

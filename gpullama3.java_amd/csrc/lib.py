@@ -57,7 +57,16 @@ def _declare(lib):
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, F, F, P, P],
-        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, P],
+        "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
+        "gl3_concat_rows": [P, P, P, I, I, I, P],
+        "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P],
+        "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P],
+        "gl3_tanh_rows": [P, P, I, L, P],
+        "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, P],
+        "gl3_shift_mix": [P, I, I, P, I, P, L, P, P, P, P, I, I, I, P],
+        "gl3_timemix": [P, P, P, P, P, P, L, L, P, P, P, I, I, I, P],
+        "gl3_head_norm_gate": [P, P, P, F, P, I, I, I, I, P],
         "gl3_kv_write": [P, I, L, I, I, P, P, P, I, P, P, I, I, I, I, I, P],
         "gl3_residual_inject": [P, P, P, I, I, P],
         "gl3_delta_state_floats": [I, I, I, I, I],
@@ -381,10 +390,11 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu", act_limit
 
 
 def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
-                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None):
+                      page_size, window, scale, v_head_dim=None, slopes=None, sink=None, keep_first=0):
     """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries. ``v_head_dim``: the values'
     size where it is not the keys'; ``slopes``: float32 [H], score - slopes[h] * distance; ``sink``: the score of a
-    key without a value that every query sees (None: no such key)."""
+    key without a value that every query sees (None: no such key); ``keep_first``: with a window, the sequence's
+    first keys that stay visible to every later query."""
     _dev(q, "q", contiguous=False); _dev(out, "out", contiguous=False)
     _dev(k_cache, "k_cache", q.dtype); _dev(v_cache, "v_cache", q.dtype)
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
@@ -405,7 +415,8 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
     _check(library().gl3_attention_generic(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
-        int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0), _stream()),
+        int(window or 0), float(scale), vd, _ptr(slopes), int(sink is not None), float(sink or 0.0),
+        int(keep_first or 0) if window else 0, _stream()),
         "attention_generic")
 
 
@@ -442,6 +453,141 @@ def residual_inject(x, rows=None, vec=None):
             raise KernelError(f"residual_inject: a vector {tuple(vec.shape)} for rows of {x.shape[1]}")
     _check(library().gl3_residual_inject(_ptr(x), _ptr(rows), _ptr(vec), x.shape[0], x.shape[1], _stream()),
            "residual_inject")
+
+
+# ------------------------------------------------------------------ around and inside mixers with a state per sequence
+def pair_rows(token_ids, positions, seq_of_token, cu_seqlens, slot_ids, state, mul_prev, mul_cur, buckets, rows):
+    """rows[t] = (previous token * mul_prev + token * mul_cur) mod buckets, ``buckets`` for a sequence's first token;
+    ``state`` [slots, >= 1] int32 holds every sequence's last token and is brought up to date."""
+    for t, n in ((token_ids, "token_ids"), (positions, "positions"), (seq_of_token, "seq_of_token"),
+                 (cu_seqlens, "cu_seqlens"), (slot_ids, "slot_ids"), (state, "state"), (rows, "rows")):
+        _dev(t, n, torch.int32)
+    T = token_ids.numel()
+    if positions.numel() != T or seq_of_token.numel() != T or rows.numel() != T or state.dim() != 2 \
+            or cu_seqlens.numel() != slot_ids.numel() + 1:
+        raise KernelError(f"pair_rows: {T} tokens, {positions.numel()} positions, state {tuple(state.shape)}")
+    _check(library().gl3_pair_rows(_ptr(token_ids), _ptr(positions), _ptr(seq_of_token), _ptr(cu_seqlens), _ptr(slot_ids),
+                                   _ptr(state), state.stride(0), int(mul_prev), int(mul_cur), int(buckets), _ptr(rows), T,
+                                   _stream()), "pair_rows")
+
+
+def concat_rows(a, b, out):
+    """out[t] = [a[t]; b[t]] in ``out``'s dtype (a, b float32 [T, d]; out [T, 2 d])."""
+    _dev(a, "a", torch.float32); _dev(b, "b", torch.float32); _dev(out, "out")
+    if a.dim() != 2 or a.shape != b.shape or out.shape != (a.shape[0], 2 * a.shape[1]):
+        raise KernelError(f"concat_rows: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_concat_rows(_ptr(a), _ptr(b), _ptr(out), _code(out, "out"), a.shape[0], a.shape[1], _stream()),
+           "concat_rows")
+
+
+def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, gate_col=0):
+    """Runs of heads inside ``rows`` [T, ld] turned in place by the tokens' positions. ``runs``: up to three of
+    ``(first column, heads, head_dim, rot_dim, cos, sin)`` with tables [positions, rot_dim / 2] float32 (None, None: not
+    rotated). ``back``: by minus the angle. ``gate`` (one run): rows [T, *] of the same dtype whose column
+    ``gate_col + h`` holds head h's gate; every element of the head is multiplied by its sigmoid."""
+    _dev(rows, "rows", contiguous=False); _dev(positions, "positions", torch.int32)
+    T = rows.shape[0]
+    if rows.dim() != 2 or rows.stride(1) != 1 or positions.numel() != T or not 1 <= len(runs) <= 3:
+        raise KernelError(f"rotate_heads: rows {tuple(rows.shape)}, {positions.numel()} positions, {len(runs)} runs")
+    n = len(runs)
+    for col, heads, hd, rd, cos, sin in runs:
+        if cos is not None:
+            _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
+            if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rd // 2:
+                raise KernelError(f"rotate_heads: table {tuple(cos.shape)} for {rd} rotated elements")
+        if col < 0 or col + heads * hd > rows.shape[1] or rd > hd or rd % 2:
+            raise KernelError(f"rotate_heads: {heads} heads of {hd} ({rd} rotated) from column {col} of rows of {rows.shape[1]}")
+    ints = [(c_int * n)(*[int(r[i]) for r in runs]) for i in range(4)]
+    tabs = [(c_void_p * n)(*[r[i].data_ptr() if r[i] is not None else None for r in runs]) for i in (4, 5)]
+    gate_ld = 0
+    if gate is not None:
+        _dev(gate, "gate", rows.dtype, contiguous=False)
+        if gate.dim() != 2 or gate.shape[0] != T or gate.stride(1) != 1 or n != 1 or gate_col < 0 or gate_col + runs[0][1] > gate.shape[1]:
+            raise KernelError(f"rotate_heads: gate {tuple(gate.shape)} from column {gate_col}")
+        gate_ld = gate.stride(0)
+    _check(library().gl3_rotate_heads(_ptr(rows), _code(rows, "rows"), rows.stride(0), _ptr(positions), T, *ints, *tabs, n,
+                                      int(bool(adjacent)), int(bool(back)), _ptr(gate), gate_ld, int(gate_col), _stream()),
+           "rotate_heads")
+
+
+def sides_norm_add(x, a, b, wa, wb, eps, factor):
+    """x += factor * (a / rms(a) * wa + b / rms(b) * wb); all float32, a and b [T, d] like x (b may be None)."""
+    _dev(x, "x", torch.float32); _dev(a, "a", torch.float32); _dev(wa, "wa", torch.float32)
+    if x.dim() != 2 or a.shape != x.shape or wa.shape != (x.shape[1],):
+        raise KernelError(f"sides_norm_add: x {tuple(x.shape)}, a {tuple(a.shape)}, weight {tuple(wa.shape)}")
+    if b is not None:
+        _dev(b, "b", torch.float32); _dev(wb, "wb", torch.float32)
+        if b.shape != x.shape or wb.shape != wa.shape:
+            raise KernelError(f"sides_norm_add: b {tuple(b.shape)}, weight {tuple(wb.shape)}")
+    _check(library().gl3_sides_norm_add(_ptr(x), _ptr(a), _ptr(b), _ptr(wa), _ptr(wb) if b is not None else c_void_p(0),
+                                        float(eps), float(factor), x.shape[0], x.shape[1], _stream()), "sides_norm_add")
+
+
+def tanh_rows(src, out):
+    """out = tanh(src) in ``out``'s dtype (src float32, same number of elements, both contiguous)."""
+    _dev(src, "src", torch.float32); _dev(out, "out")
+    if src.numel() != out.numel():
+        raise KernelError(f"tanh_rows: {src.numel()} inputs for {out.numel()} outputs")
+    _check(library().gl3_tanh_rows(_ptr(src), _ptr(out), _code(out, "out"), src.numel(), _stream()), "tanh_rows")
+
+
+def mingru_scan(proj, width, state, cu_seqlens, slot_ids, out):
+    """The minGRU recurrence over the step's tokens from the state in each sequence's slot: ``proj`` [T, >= 3 width]
+    float32 holds the update gate's, the candidate's and the output gate's sums; ``out`` [T, width] receives
+    S_t * silu(gate); ``state`` [slots, >= width] float32 is advanced."""
+    _dev(proj, "proj", torch.float32, contiguous=False); _dev(state, "state", torch.float32, contiguous=False); _dev(out, "out")
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
+    T, B = proj.shape[0], slot_ids.numel()
+    if (state.dim() != 2 or state.stride(1) != 1 or proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < 3 * width or out.shape != (T, width) or state.dim() != 2
+            or state.shape[1] < width or cu_seqlens.numel() != B + 1):
+        raise KernelError(f"mingru_scan: proj {tuple(proj.shape)}, out {tuple(out.shape)}, state {tuple(state.shape)}")
+    _check(library().gl3_mingru_scan(_ptr(proj), proj.stride(0), int(width), _ptr(state), state.stride(0), _ptr(cu_seqlens),
+                                     _ptr(slot_ids), _ptr(out), _code(out, "out"), B, _stream()), "mingru_scan")
+
+
+def shift_mix(h, mu, state, cu_seqlens, seq_of_token, slot_ids, out, one_token_each=False):
+    """out[s, t] = h[t] + (row of the token before t - h[t]) * mu[s]; a step's first token of a sequence reads the row
+    that ``state`` [slots, >= d] float32 holds for it, and the step's last row is left there. ``mu`` [n, d] float32;
+    ``out`` [n, T, d] of h's dtype."""
+    _dev(h, "h"); _dev(mu, "mu", torch.float32); _dev(state, "state", torch.float32, contiguous=False); _dev(out, "out", h.dtype)
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
+    _dev(slot_ids, "slot_ids", torch.int32)
+    T, d = h.shape
+    B = slot_ids.numel()
+    if (mu.dim() != 2 or mu.shape[1] != d or out.shape != (mu.shape[0], T, d) or state.dim() != 2 or state.shape[1] < d
+            or state.stride(1) != 1
+            or cu_seqlens.numel() != B + 1 or seq_of_token.numel() != T):
+        raise KernelError(f"shift_mix: h {tuple(h.shape)}, mu {tuple(mu.shape)}, out {tuple(out.shape)}, state {tuple(state.shape)}")
+    _check(library().gl3_shift_mix(_ptr(h), _code(h, "h"), d, _ptr(mu), mu.shape[0], _ptr(state), state.stride(0),
+                                   _ptr(cu_seqlens), _ptr(seq_of_token), _ptr(slot_ids), _ptr(out), T, B,
+                                   int(bool(one_token_each)), _stream()), "shift_mix")
+
+
+def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, H, D):
+    """The decayed matrix per head, token by token from the state in each sequence's slot (``mixers.hip``): r, k, v,
+    w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D]; ``out`` [T, H D] float32 receives the raw
+    read-outs; ``state`` [slots, >= state_off + H D D] float32."""
+    for t, n in ((r, "r"), (k, "k"), (v, "v"), (w_log, "w_log"), (bonus, "bonus"), (out, "out")):
+        _dev(t, n, torch.float32)
+    _dev(state, "state", torch.float32, contiguous=False)
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
+    T, B = r.shape[0], slot_ids.numel()
+    if (any(t.shape != (T, H * D) for t in (r, k, v, w_log, out)) or bonus.numel() != H * D or state.dim() != 2
+            or state.shape[1] < state_off + H * D * D or state.stride(1) != 1 or cu_seqlens.numel() != B + 1):
+        raise KernelError(f"timemix: r {tuple(r.shape)} for {H} heads of {D}, state {tuple(state.shape)}")
+    _check(library().gl3_timemix(_ptr(r), _ptr(k), _ptr(v), _ptr(w_log), _ptr(bonus), _ptr(state), state.stride(0),
+                                 int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out), B, H, D, _stream()), "timemix")
+
+
+def head_norm_gate(o, weight, gate, eps, out, H, D):
+    """out[t, h] = o[t, h] / rms(o[t, h]) * weight[h] * silu(gate[t, h]) per head of D elements; o, gate [T, H D] float32,
+    weight [H D] float32, out [T, H D]."""
+    _dev(o, "o", torch.float32); _dev(weight, "weight", torch.float32); _dev(gate, "gate", torch.float32); _dev(out, "out")
+    T = o.shape[0]
+    if o.shape != (T, H * D) or gate.shape != o.shape or out.shape != o.shape or weight.numel() != H * D:
+        raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, gate {tuple(gate.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_head_norm_gate(_ptr(o), _ptr(weight), _ptr(gate), float(eps), _ptr(out), _code(out, "out"), T, H, D,
+                                        _stream()), "head_norm_gate")
 
 
 # ------------------------------------------------------------------ the gated delta rule

@@ -10,7 +10,12 @@ projections have no biases; a description that names ``q_bias``, ``k_bias``, ``v
 What other decoders' descriptions may ask for besides: no rotation (``position`` None), values of another size than
 the keys (``v_head_dim``), a bias on the scores that grows with the distance (``distance_bias``: a slope per head), a
 sink in the softmax (``sink``), and a learned factor per channel on the output (``out_scale_name``), applied by the
-output projection's epilogue.
+output projection's epilogue; a window that keeps a sequence's first positions visible (``keep_first``); values that
+are rotated by their own position before they are cached, with every head's output turned back by the query's
+position (``value_position``); a gate per head (``head_gate`` among the names: sigmoid of one more row per head of the
+stacked projection, multiplied into the head's output); a constant factor on the output (``out_mult``). The last three
+run on kernels that take any head sizes: one product, one kernel that turns q, k and v in place, the cache write, the
+attention, one kernel that turns the output back and applies the gate.
 """
 from __future__ import annotations
 
@@ -39,9 +44,17 @@ class GQAAttention:
         # zero rows (q, k, v) and zero columns (o) up to the next multiple of 16: scores and outputs are the same
         # numbers, and every kernel sees the padded sizes.
         self.hs_stored, self.vd_stored = self.hs, self.vd
-        if spec.position is None:
+        self.value_position_spec = getattr(spec, "value_position", None)
+        self.gated = "head_gate" in spec.names
+        # (rotated values, a gate per head, and a rotation with values of another size run on the kernels for any sizes)
+        self.general = bool(self.value_position_spec is not None or self.gated
+                            or (spec.position is not None and self.vd != self.hs))
+        if spec.position is None or self.general:
+            # (a rotation touches a head's first elements only: zeros behind them stay zeros)
             self.hs, self.vd = -(-self.hs // 16) * 16, -(-self.vd // 16) * 16
         self.window = spec.window
+        self.keep_first = int(getattr(spec, "keep_first", 0) or 0) if spec.window else 0
+        self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.sink = getattr(spec, "sink", None)
         bias = getattr(spec, "distance_bias", None)
         self._slopes_host = bias.slopes(self.H) if bias is not None else None
@@ -51,6 +64,10 @@ class GQAAttention:
         self.out_scale = None
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(self.hs)
         self.position = build_part("position", spec.position, device=device) if spec.position is not None else None
+        self.value_position = (build_part("position", self.value_position_spec, device=device)
+                               if self.value_position_spec is not None else None)
+        if self.value_position is not None and self.value_position.rot_dim > self.vd_stored:
+            raise ValueError(f"values of {self.vd_stored} elements cannot be rotated over {self.value_position.rot_dim}")
         self.names = spec.names
         self.biased = "q_bias" in self.names
         if self.biased and not ("k_bias" in self.names and "v_bias" in self.names):
@@ -69,12 +86,16 @@ class GQAAttention:
             out[n["o_bias"]] = TensorSpec((d,), "vector", 0.0, 0.1)
         if self.out_scale_name:
             out[self.out_scale_name] = TensorSpec((d,), "vector", 1.0, 0.1)
+        if self.gated:
+            out[n["head_gate"]] = TensorSpec((self.H, d))
         return out
 
     def load(self, weights):
         n = self.names
         if (self.hs, self.vd) != (self.hs_stored, self.vd_stored):
             weights = _PaddedHeads(weights, self)
+        if self.general:
+            return self._load_general(weights)
         parts = [weights[n["q"]], weights[n["k"]], weights[n["v"]]]
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         self.w_qkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
@@ -105,21 +126,54 @@ class GQAAttention:
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
         if "o_bias" in n:
             self.b_o = weights[n["o_bias"]].float().contiguous()
+        self._load_scales(weights)
+        if self._slopes_host is not None:
+            self.slopes = torch.tensor(self._slopes_host, dtype=torch.float64).to(torch.float32).to(self.w_qkv.device)
+
+    def _load_scales(self, weights):
         if self.out_scale_name:
             self.out_scale = weights[self.out_scale_name].float().contiguous()
+        if self.out_mult != 1.0:      # the constant rides in the output projection's epilogue with the factor per channel
+            dev = weights[self.names["o"]].device
+            self.out_scale = (self.out_scale * self.out_mult if self.out_scale is not None
+                              else torch.full((self.d,), self.out_mult, dtype=torch.float32, device=dev))
+
+    def _load_general(self, weights):
+        """q, k, v and the heads' gates stacked for one product (zero rows up to a multiple of 16), stored order."""
+        n = self.names
+        if self.biased or "o_bias" in n:
+            raise ValueError("an attention with rotated values or a gate per head is built without biases")
+        parts = [weights[n[k]] for k in ("q", "k", "v")] + ([weights[n["head_gate"]]] if self.gated else [])
+        dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
+        rows = sum(p.shape[0] for p in parts)
+        pad = torch.zeros((-(-rows // 16) * 16 - rows, self.d), dtype=dt, device=parts[0].device)
+        self.w_qkv = torch.cat([p.to(dt) for p in parts] + [pad], dim=0).contiguous()
+        lo = 0
+        for k, p in zip(("q", "k", "v", "head_gate"), parts):      # the stored names stay addressable as views
+            weights[n[k]] = self.w_qkv[lo:lo + p.shape[0]]
+            lo += p.shape[0]
+        without = getattr(self, "without", frozenset())
+        ops.for_few_rows(self.w_qkv, without=without)
+        self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
+        self._load_scales(weights)
         if self._slopes_host is not None:
             self.slopes = torch.tensor(self._slopes_host, dtype=torch.float64).to(torch.float32).to(self.w_qkv.device)
 
     def kv_need(self):
-        return KVNeed(self.Kh, self.hs, self.window, v_head_dim=None if self.vd == self.hs else self.vd)
+        return KVNeed(self.Kh, self.hs, self.window, v_head_dim=None if self.vd == self.hs else self.vd,
+                      keep_first=self.keep_first)
 
     def state_need(self):
         return None
 
-    def forward(self, ctx, h, x, run):
+    def forward(self, ctx, h, x, run, epilogue=ops.EPI_ADD):
+        """``epilogue``: EPI_ADD adds the output into the residual rows ``x``; EPI_STORE writes it to ``x``, a float32
+        buffer of the caller's (a mixer that stands beside another)."""
         T, H, Kh, hs, vd = h.shape[0], self.H, self.Kh, self.hs, self.vd
         k_cache, v_cache = ctx.cache.layer_kv(run.kv_entry)
         table = ctx.block_table(ctx.cache.group_index(run.kv_entry))
+        if self.general:
+            return self._forward_general(ctx, h, x, run, epilogue, k_cache, v_cache, table)
         if vd == hs:
             q = ops.qkv_project(ctx, h, self.w_qkv, self.w_q, self.position, k_cache, v_cache, table, H, Kh, hs,
                                 self.dtype, run.writes_kv, bias=self.b_qkv)
@@ -127,8 +181,37 @@ class GQAAttention:
             q = self._project_unequal(ctx, h, k_cache, v_cache, table, run)
         att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
         ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
-                      slopes=self.slopes, sink=self.sink)
-        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx, bias=self.b_o, col_scale=self.out_scale)
+                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first)
+        ops.linear(att, self.w_o, x, epilogue, ctx, bias=self.b_o, col_scale=self.out_scale)
+
+    def _forward_general(self, ctx, h, x, run, epilogue, k_cache, v_cache, table):
+        if not run.writes_kv:
+            raise ValueError("an attention with rotated values or a gate per head keeps keys and values of its own")
+        T, H, Kh, hs, vd = h.shape[0], self.H, self.Kh, self.hs, self.vd
+        qn, kn, vn = H * hs, Kh * hs, Kh * vd
+        qkv = ctx.buffer("qkvg", (T, self.w_qkv.shape[0]), self.dtype)
+        ops.linear(h, self.w_qkv, qkv, ops.EPI_STORE, ctx)
+        pos, vpos = self.position, self.value_position
+        runs = []
+        if pos is not None:
+            runs += [(0, H, hs, pos.rot_dim, pos.cos, pos.sin), (qn, Kh, hs, pos.rot_dim, pos.cos, pos.sin)]
+        if vpos is not None:
+            runs.append((qn + kn, Kh, vd, vpos.rot_dim, vpos.cos, vpos.sin))
+        if runs:
+            K.rotate_heads(qkv, ctx.positions, runs, adjacent=bool((pos or vpos).adjacent))
+        K.kv_write(qkv, qn, qn + kn, ctx.positions, ops._table_rows(ctx), table, k_cache, v_cache, Kh, hs, vd,
+                   k_cache.shape[2])
+        att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
+        ops.attention(ctx, qkv, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
+                      slopes=self.slopes, sink=self.sink, keep_first=self.keep_first)
+        if vpos is not None or self.gated:
+            # every head's output turned back by the query's position, then times the head's gate
+            K.rotate_heads(att, ctx.positions,
+                           [(0, H, vd, vpos.rot_dim if vpos is not None else 0, vpos.cos if vpos is not None else None,
+                             vpos.sin if vpos is not None else None)],
+                           adjacent=bool(vpos is not None and vpos.adjacent), back=True,
+                           gate=qkv if self.gated else None, gate_col=qn + kn + vn)
+        ops.linear(att, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)
 
     def _project_unequal(self, ctx, h, k_cache, v_cache, table, run):
         """Values of another size than the keys: one product over the stacked rows, then keys and values into the

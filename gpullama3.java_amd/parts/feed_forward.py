@@ -29,6 +29,7 @@ class GatedFeedForward:
         self.up_shift = float(getattr(spec, "up_shift", 0.0))
         self.out_scale_name = getattr(spec, "out_scale_name", None)
         self.out_scale = None
+        self.out_mult = float(getattr(spec, "out_mult", 1.0))
         self.biased = "gate_bias" in self.names
         if self.biased != ("up_bias" in self.names):
             raise ValueError("a gated feed-forward names the biases of gate and up together or neither")
@@ -70,6 +71,9 @@ class GatedFeedForward:
             self.b_down = weights[n["down_bias"]].float().contiguous()
         if self.out_scale_name:
             self.out_scale = weights[self.out_scale_name].float().contiguous()
+        if self.out_mult != 1.0:      # the constant rides in the down projection's epilogue with the factor per channel
+            self.out_scale = (self.out_scale * self.out_mult if self.out_scale is not None
+                              else torch.full((self.d,), self.out_mult, dtype=torch.float32, device=self.w_down.device))
 
     def folds_norm(self, h):
         """Whether the first product takes over the work of the norm that ``h`` (an ``ops.Normed``) stands for."""

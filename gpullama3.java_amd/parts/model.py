@@ -9,6 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..csrc import lib as K
+from ..cache import StateNeed
 from ..weights.loader import TensorSpec
 from . import ops
 from .base import RunInfo, build_part
@@ -26,6 +27,7 @@ def expected_tensors(spec, dtype=torch.float32, device="cpu"):
     if spec.final_norm is not None:
         out.update(_norm_tensors(spec.final_norm))
     out.update(_inject_tensors(spec))
+    out.update(_around_tensors(spec))
     for b in spec.layers:
         block = build_part("block", b, dtype=dtype, device=device)
         for p in block.parts():
@@ -46,12 +48,26 @@ def _block_needs(block):
     return (keepers[0].kv_need(), keepers[0].state_need()) if keepers else (None, None)
 
 
+def _around_tensors(spec):
+    """What stands around the blocks beside embedding, head and final norm: the table of token pairs, and the matrices
+    that mix the residual rows with the embedding's output in front of a run-order entry."""
+    out = {}
+    pair = getattr(spec, "pair_embedding", None)
+    if pair is not None:
+        out[pair.table_name] = TensorSpec((pair.buckets + 1, spec.hidden))
+    for r in spec.run_order:
+        b = getattr(r, "before", None)
+        if b is not None and hasattr(b, "weight_name"):
+            out[b.weight_name] = TensorSpec((spec.hidden, 2 * spec.hidden))
+    return out
+
+
 def _inject_tensors(spec):
     """The tables of vectors that entries of the run order add to the residual rows before they run."""
     out = {}
     for r in spec.run_order:
         b = getattr(r, "before", None)
-        if b is not None and b.vector_name is not None:
+        if b is not None and getattr(b, "vector_name", None) is not None:
             if not 0 <= b.row < b.vector_rows:
                 raise ValueError(f"a run-order entry adds row {b.row} of {b.vector_name!r}, which has {b.vector_rows}")
             out[b.vector_name] = TensorSpec((b.vector_rows, spec.hidden), "matrix")
@@ -101,6 +117,7 @@ class DecoderModel:
         if self.final_norm is not None:
             out.update(self.final_norm.tensors())
         out.update(_inject_tensors(self.spec))
+        out.update(_around_tensors(self.spec))
         for b in self.blocks:
             for p in b.parts():
                 out.update(p.tensors())
@@ -126,8 +143,16 @@ class DecoderModel:
             self.final_norm.load(weights)
         # what entries of the run order add to the residual rows, which are 32-bit: the vectors in 32-bit
         self.inject_vectors = {name: weights[name].float().contiguous() for name in _inject_tensors(self.spec)}
-        self.keeps_embedding = any(getattr(r, "before", None) is not None and r.before.embedding
+        self.keeps_embedding = any(getattr(r, "before", None) is not None
+                                   and (getattr(r.before, "embedding", False) or hasattr(r.before, "weight_name"))
                                    for r in self.spec.run_order)
+        pair = getattr(self.spec, "pair_embedding", None)
+        self.pair_table = weights[pair.table_name].to(self.embedding.dtype) if pair is not None else None
+        self.remix = {}
+        for r in self.spec.run_order:
+            b = getattr(r, "before", None)
+            if b is not None and hasattr(b, "weight_name") and b.weight_name not in self.remix:
+                self.remix[b.weight_name] = ops.for_few_rows(weights[b.weight_name], without=self.without)
         for b in self.blocks:
             for p in b.parts():
                 p.load(weights)
@@ -138,6 +163,10 @@ class DecoderModel:
             kv_need, state_need = _block_needs(self.blocks[r.layer])
             kv.append(kv_need if run.writes_kv else None)
             state.append(state_need)
+        if getattr(self.spec, "pair_embedding", None) is not None:
+            # one more state area behind the run order's: every sequence's last token, for the table of token pairs
+            kv.append(None)
+            state.append(StateNeed(1, torch.int32))
         return kv, state
 
     def forward(self, ctx, want_rows):
@@ -153,6 +182,16 @@ class DecoderModel:
             around["scale"] = self.spec.embedding_scale
         if self.position_table is not None:
             around.update(pos_table=self.position_table, positions=ctx.positions)
+        pair = getattr(self.spec, "pair_embedding", None)
+        if pair is not None:
+            # the row of the pair table per token (the embedding kernel adds a row of a second table by index: here the
+            # index is the pair's hash, not the position); the sequences' last tokens move on in their slots
+            if self.position_table is not None:
+                raise ValueError("a decoder has learned positions or a table of token pairs, not both")
+            pair_rows = ctx.buffer("pair_rows", (ctx.n_tokens,), torch.int32)
+            K.pair_rows(ctx.token_ids, ctx.positions, ctx.seq_of_token, ctx.cu_seqlens, ctx.slot_ids,
+                        ctx.cache.slot_state(len(self.runs)), pair.mul_prev, pair.mul_cur, pair.buckets, pair_rows)
+            around.update(pos_table=self.pair_table, positions=pair_rows)
         if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS and getattr(firsts[0], "folds", False):
             # the first norm's sums of squares, and its rows times its weight, come with the embedding
             ssq = ctx.ssq_buffer(1)
@@ -169,7 +208,14 @@ class DecoderModel:
             K.embed(self.embedding, ctx.token_ids, embedded, **around)
         for i, (run, block) in enumerate(zip(self.runs, order)):
             before = getattr(self.spec.run_order[i], "before", None)
-            if before is not None:
+            if before is not None and hasattr(before, "weight_name"):
+                # x <- W [x; x0]: the rows and the embedding's output side by side as the product's input
+                ops.settle_residual(ctx, x)
+                both = ctx.buffer("rows_and_embedding", (ctx.n_tokens, 2 * self.spec.hidden), self.dtype)
+                K.concat_rows(x, embedded, both)
+                ops.linear(both, self.remix[before.weight_name], x, ops.EPI_STORE, ctx)
+                ops.residual_written(ctx, x)
+            elif before is not None:
                 ops.settle_residual(ctx, x)
                 vec = self.inject_vectors[before.vector_name][before.row] if before.vector_name is not None else None
                 K.residual_inject(x, embedded if before.embedding else None, vec)

@@ -457,12 +457,17 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
 
 
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale, v_head_dim=None,
-              slopes=None, sink=None):
+              slopes=None, sink=None, keep_first=0):
     """``v_head_dim``: the values' size (None: the keys'); ``slopes``: float32 [H], a bias of -slopes[h] * distance
-    on the scores; ``sink``: the score of a key without a value that every query sees (None: none)."""
+    on the scores; ``sink``: the score of a key without a value that every query sees (None: none); ``keep_first``:
+    with a window, the sequence's first keys that every later query still sees."""
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     disabled = _off(ctx)
     extras = dict(slopes=slopes, sink=sink)
+    keep_first = int(keep_first or 0) if window else 0
+    if keep_first:
+        return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
+                                   head_dim, page, window, scale, v_head_dim=v_head_dim, keep_first=keep_first, **extras)
     if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):

@@ -23,7 +23,9 @@ def frequencies(head_dim, theta, scaling):
     out = np.zeros(head_dim // 2, dtype=_F)
     for n, i in enumerate(range(0, head_dim, 2)):
         freq = _F(1.0 / math.pow(theta, i / head_dim))
-        if scaling is not None:
+        if scaling is not None and not hasattr(scaling, "low_freq_factor"):
+            freq = _F(freq / _F(scaling.factor))          # linear scaling: every frequency divided alike
+        elif scaling is not None:
             factor, lo, hi = _F(scaling.factor), _F(scaling.low_freq_factor), _F(scaling.high_freq_factor)
             old = _F(scaling.original_max_position)
             wavelen = _F(2.0 * math.pi / float(freq))

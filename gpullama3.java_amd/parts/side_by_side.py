@@ -1,0 +1,94 @@
+"""Two mixers side by side: both read the same normalised input, each one's output is normalised over the model width
+with a weight of its own, and ``weight`` times the sum of the two (1/2: their average) is the mixer's output.
+
+Either side is any registered mixer whose ``forward`` takes ``epilogue=ops.EPI_STORE`` (its output then goes to a
+float32 buffer instead of into the residual rows). Keys and values are the one side's that asks for them; states of
+both sides share the run-order entry's state area, the left side's first.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache import StateNeed
+from ..csrc import lib as K
+from ..weights.loader import TensorSpec
+from . import ops
+from .base import build_part, register_part
+
+
+class _Shifted:
+    """A step context whose per-slot state is a side's own columns of the entry's state area."""
+
+    def __init__(self, ctx, lo, hi):
+        self.__dict__["_ctx"], self.__dict__["_lo"], self.__dict__["_hi"] = ctx, lo, hi
+
+    def __getattr__(self, name):
+        return getattr(self._ctx, name)
+
+    def __setattr__(self, name, value):
+        setattr(self._ctx, name, value)
+
+    def slot_state(self, entry):
+        return self._ctx.slot_state(entry)[:, self._lo:self._hi]
+
+
+class SideBySide:
+    adds_only = True       # never reads the residual rows
+
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+        self.d, self.names = spec.hidden, spec.names
+        self.left = build_part("mixer", spec.left, dtype=dtype, device=device)
+        self.right = build_part("mixer", spec.right, dtype=dtype, device=device)
+        self.factor = float(spec.weight) * float(getattr(spec, "out_mult", 1.0))
+        self.w_left = self.w_right = None
+        needs = [s.state_need() for s in (self.left, self.right)]
+        if any(n is not None and n.dtype != torch.float32 for n in needs):
+            raise ValueError("mixers side by side keep their states in 32-bit floats")
+        self.state_sizes = [0 if n is None else -(-n.elements // 4) * 4 for n in needs]
+        if sum(1 for s in (self.left, self.right) if s.kv_need() is not None) > 1:
+            raise ValueError("of two mixers side by side at most one keeps keys and values")
+
+    @property
+    def graph_safe(self):
+        return bool(getattr(self.left, "graph_safe", False) and getattr(self.right, "graph_safe", False))
+
+    def tensors(self):
+        out = {self.names["left_norm"]: TensorSpec((self.d,), "vector"), self.names["right_norm"]: TensorSpec((self.d,), "vector")}
+        out.update(self.left.tensors())
+        out.update(self.right.tensors())
+        return out
+
+    def load(self, weights):
+        for side in (self.left, self.right):
+            side.without = getattr(self, "without", frozenset())
+            side.may_hold_once = getattr(self, "may_hold_once", False)
+            side.load(weights)
+        self.w_left = weights[self.names["left_norm"]].float().contiguous()
+        self.w_right = weights[self.names["right_norm"]].float().contiguous()
+
+    def kv_need(self):
+        return self.left.kv_need() or self.right.kv_need()
+
+    def state_need(self):
+        n = sum(self.state_sizes)
+        return StateNeed(n, torch.float32) if n else None
+
+    def forward(self, ctx, h, x, run):
+        if isinstance(h, ops.Normed):
+            h = h.materialize()
+        T = h.shape[0]
+        next_norm, ctx.next_norm = ctx.next_norm, None      # neither side completes the residual rows
+        outs, lo = [], 0
+        for name, side, size in (("left", self.left, self.state_sizes[0]), ("right", self.right, self.state_sizes[1])):
+            out = ctx.buffer(f"side_{name}", (T, self.d), torch.float32)
+            side.forward(_Shifted(ctx, lo, lo + size) if size else ctx, h, out, run, epilogue=ops.EPI_STORE)
+            outs.append(out)
+            lo += size
+        ctx.next_norm = next_norm
+        ops.settle_residual(ctx, x)
+        K.sides_norm_add(x, outs[0], outs[1], self.w_left, self.w_right, self.spec.norm_eps, self.factor)
+        ops.residual_written(ctx, x)
+
+
+register_part("mixer", "side_by_side", SideBySide)
