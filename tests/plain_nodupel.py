@@ -182,9 +182,9 @@ class Sequence:
             self.layers.append(x.copy())
         self.n += T
         self.prev_token = tokens[-1]
-        cap = cfg["logit_softcap"]
+        cap = cfg.get("logit_softcap")
         logits = linear(rms_norm(x, W["final.norm"], eps), W["head"])
-        return cap * np.tanh(logits / cap)
+        return logits if cap is None else cap * np.tanh(logits / cap)
 
     def mingru(self, mc, p, h, st):
         W = self.W
@@ -234,3 +234,65 @@ class Sequence:
 def forward(cfg, W, tokens):
     """Logits [T, vocab] of one sequence from its start."""
     return Sequence(cfg, W).feed(list(tokens))
+
+
+# ----------------------------------------------------------------- weights for tests
+def tensor_shapes(cfg, decay_rank=8):
+    d = cfg["width"]
+    out = {"embed": (cfg["vocab"], d), "bigram": (cfg["embedding"]["bigram"]["buckets"] + 1, d),
+           "final.norm": (d,), "head": (cfg["vocab"], d)}
+    if cfg.get("loop"):
+        out["loop.in"] = (d, 2 * d)
+    for i, lay in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        out[p + "norm1"] = (d,)
+        m = lay["mixer"]
+        if lay["type"] == "mingru":
+            w = m["width"]
+            out.update({p + "mix.z": (w, d), p + "mix.z.b": (w,), p + "mix.x": (w, d), p + "mix.x.b": (w,),
+                        p + "mix.g": (w, d), p + "mix.o": (d, w)})
+        else:
+            L, R = m["left"], m["right"]
+            q = p + "mix.left."
+            out.update({q + "q": (L["heads"] * L["dim"], d), q + "k": (L["kv_heads"] * L["dim"], d),
+                        q + "v": (L["kv_heads"] * L["vdim"], d), q + "g": (L["heads"], d),
+                        q + "o": (d, L["heads"] * L["vdim"]), q + "out": (d,)})
+            r = p + "mix.right."
+            hd = R["heads"] * R["dim"]
+            out.update({r + "mu." + s: (d,) for s in "rkvgw"})
+            out.update({r + s: (hd, d) for s in "rkvg"})
+            out.update({r + "w1": (decay_rank, d), r + "w2": (hd, decay_rank), r + "w0": (hd,), r + "u": (R["heads"], R["dim"]),
+                        r + "norm": (hd,), r + "o": (d, hd), r + "out": (d,)})
+        if lay.get("mlp") is not None:
+            ff = lay["mlp"]["ff"]
+            out.update({p + "norm2": (d,), p + "mlp.gate": (ff, d), p + "mlp.up": (ff, d), p + "mlp.down": (d, ff)})
+    return out
+
+
+def make_weights(cfg, seed, decay_rank=8):
+    """float32 weights that bfloat16 holds exactly, sized so that every mechanism moves the logits: matrices
+    N(0, 1.5/sqrt(fan-in)), norm weights around one, blends anywhere between the two tokens, a wide spread of decays."""
+    import zlib
+    import torch
+    out = {}
+    for name, shape in tensor_shapes(cfg, decay_rank).items():
+        rng = np.random.default_rng([seed, zlib.crc32(name.encode())])
+        last = name.split(".")[-1]
+        if last in ("norm1", "norm2", "norm", "out"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif ".mu." in name:
+            a = rng.uniform(0.0, 1.0, shape)
+        elif last == "w0":
+            a = rng.uniform(-5.0, 0.5, shape)
+        elif last == "u" and ".right." in name:
+            a = 0.5 * rng.standard_normal(shape)
+        elif last == "b" and len(shape) == 1:
+            a = 0.5 * rng.standard_normal(shape)
+        elif name == "embed":
+            a = rng.standard_normal(shape) / cfg["embedding"]["scale"]
+        elif name == "bigram":
+            a = 0.7 * rng.standard_normal(shape)
+        else:
+            a = rng.standard_normal(shape) * (1.5 / np.sqrt(shape[-1]))
+        out[name] = torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).float().numpy()
+    return out
