@@ -63,7 +63,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits,
-    const float* __restrict__ slopes, int has_sink, float sink) {
+    const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
   constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
@@ -97,7 +97,11 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     first_pages[b] = __builtin_amdgcn_readfirstlane(bt[min(page_of((wave + b * NW) * 32), table_stride - 1)]);
   const int kv_len = __builtin_amdgcn_readfirstlane(positions[t]) + 1;
   const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
-  const int chunk_lo = lo / 32, chunk_hi = (kv_len + 31) / 32;
+  // With a window, the sequence's first keep_first keys stay visible (BIAS kernels only). Their chunks that lie before
+  // the window's first chunk are numbered in front of it: chunk_lo .. chunk_w - 1 stand for chunks 0 .. chunk_w - chunk_lo - 1.
+  const int chunk_w = lo / 32, chunk_hi = (kv_len + 31) / 32;
+  const int chunk_lo = chunk_w - (BIAS ? min((keep_first + 31) / 32, chunk_w) : 0);
+  auto real = [&](int ck) { return (BIAS && ck < chunk_w) ? ck - chunk_lo : ck; };
   const int per_split = n_splits == 1 ? chunk_hi - chunk_lo : (chunk_hi - chunk_lo + n_splits - 1) / n_splits;
   const int c_begin = chunk_lo + split * per_split;
   const int c_end = min(chunk_hi, c_begin + per_split);
@@ -123,7 +127,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     for (int b = 0; b < CB; ++b) {
       const int ck = ck0 + b * NW;
       if (ck < c_end) {
-        const int key0 = ck * 32;
+        const int key0 = real(ck) * 32;
         // (the first chunks from the sequence's start: their pages are here already)
         const long page = (c_begin == 0 && ck0 == wave) ? first_pages[b] : __builtin_amdgcn_readfirstlane(bt[page_of(key0)]);
         const int po = in_page(key0);
@@ -148,7 +152,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     for (int b = 0; b < CB; ++b) {
       const int ck = ck0 + b * NW;
       if (ck >= c_end) break;
-      const int key0 = ck * 32;
+      const int key0 = real(ck) * 32;
       f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
@@ -162,8 +166,8 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
       for (int v = 0; v < 4; ++v) {
         const int ka_i = key0 + 8 * qd + v, kb_i = ka_i + 4;
         const float da = BIAS ? slope * (float)(kv_len - 1 - ka_i) : 0.f;     // (the bias: slope * distance; 4 keys on: 4 slopes less)
-        s[v] = (ka_i >= lo && ka_i < kv_len) ? sa[v] * scale - da : -INFINITY;
-        s[4 + v] = (kb_i >= lo && kb_i < kv_len) ? sb[v] * scale - (BIAS ? da - 4.f * slope : 0.f) : -INFINITY;
+        s[v] = ((ka_i >= lo || (BIAS && ka_i < keep_first)) && ka_i < kv_len) ? sa[v] * scale - da : -INFINITY;
+        s[4 + v] = ((kb_i >= lo || (BIAS && kb_i < keep_first)) && kb_i < kv_len) ? sb[v] * scale - (BIAS ? da - 4.f * slope : 0.f) : -INFINITY;
         mx = fmaxf(mx, fmaxf(s[v], s[4 + v]));
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -319,7 +323,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                                     int table_stride, float* part_o, float* part_ml, long part_floats, void* out,
                                     long out_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
                                     int window, float scale, int n_splits, const float* slopes, int has_sink, float sink,
-                                    hipStream_t stream) {
+                                    int keep_first, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && positions && block_table && out && table_stride > 0,
               "gl3_attention_decode: null argument");
@@ -344,11 +348,12 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   // More blocks than CUs: 4 waves, so that a CU holds two blocks and the second 256 blocks do not wait for the
   // first to end (what a block does before its keys arrive is a chain of trips to memory, paid once per round).
   const bool small = blocks * n_splits > 256;
-  const bool biased = slopes != nullptr || has_sink;
+  GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_decode: %d kept first keys without a window", keep_first);
+  const bool biased = slopes != nullptr || has_sink || keep_first > 0;    // (the kernels that know of kept first keys)
 #define AD_ARGS                                                                                                       \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table,    \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, n_heads / n_kv, page_size, page_shift, window,  \
-      scale, n_splits, slopes, has_sink, sink
+      scale, n_splits, slopes, has_sink, sink, keep_first
 #define GO(HS)                                                                                                        \
   do {                                                                                                                \
     constexpr int CB = HS <= 64 ? 4 : HS <= 96 ? 3 : 2;                                                               \

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
   constexpr int KROW = HS + 8;            // a key row in shared memory, in elements
@@ -77,7 +77,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   // the block's range of chunks, and the wave's own inside it
   const int blk_first = before + qb * 64, blk_last = before + min(qb * 64 + 63, q_len - 1);
   const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
-  const int ck0 = blk_lo / 32, ck1 = blk_last / 32;
+  // With a window, the sequence's first keep_first keys stay visible (BIAS kernels only). Their chunks that lie before
+  // the window's first chunk ckw are numbered in front of it: ck0 .. ckw - 1 stand for chunks 0 .. ckw - ck0 - 1.
+  const int ckw = blk_lo / 32, ck1 = blk_last / 32;
+  const int ck0 = ckw - (BIAS ? min((keep_first + 31) / 32, ckw) : 0);
+  auto real = [&](int ck) { return (BIAS && ck < ckw) ? ck - ck0 : ck; };
   const int qi0 = qb * 64 + wave * 16;     // first query of this wave, counted inside the step's tokens
   const bool active = qi0 < q_len;
   const bool q_ok = qi0 + j < q_len;
@@ -184,8 +188,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int k1 = key0 + 8 * qd + v, k2 = k1 + 4;
-        s[v] = (k1 >= lo_mine && k1 <= p_mine) ? s[v] : -INFINITY;
-        s[4 + v] = (k2 >= lo_mine && k2 <= p_mine) ? s[4 + v] : -INFINITY;
+        s[v] = ((k1 >= lo_mine || (BIAS && k1 < keep_first)) && k1 <= p_mine) ? s[v] : -INFINITY;
+        s[4 + v] = ((k2 >= lo_mine || (BIAS && k2 < keep_first)) && k2 <= p_mine) ? s[4 + v] : -INFINITY;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
@@ -215,7 +219,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 
 #pragma unroll
   for (int r = 0; r < AHEAD; ++r)
-    if (ck0 + r <= ck1) fetch(ck0 + r, rk[r], rv[r]);
+    if (ck0 + r <= ck1) fetch(real(ck0 + r), rk[r], rv[r]);
   stage(0, rk[0], rv[0]);
   __syncthreads();
   int buf = 0;
@@ -224,11 +228,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     for (int r = 0; r < AHEAD; ++r) {
       const int ck = base + r;
       if (ck > ck1) break;
-      const int key0 = ck * 32;
+      const int key0 = real(ck) * 32;
       // the registers of this chunk are free (it lies in shared memory): ask for the chunk three further;
-      fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);   // unconditional (the last chunk again at the end): a branch
+      fetch(real(min(ck + AHEAD, ck1)), rk[r], rv[r]);   // unconditional (the last chunk again at the end): a branch
                                                    // around the loads makes the compiler wait for all of them at once
-      if (ck >= ck_first && ck <= ck_last) {
+      if (active && (ck >= ck_first || (BIAS && key0 < keep_first)) && ck <= ck_last) {
         bf16x8 ka[KK], kb2[KK], vt[DT];
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vt[dt] = *(const bf16x8*)&vs[buf][dt * 16 + j][8 * qd];
         // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
-        const bool masked = !(key0 + 31 <= p_first && key0 >= lo_last);
+        const bool masked = (BIAS && ck < ckw) || !(key0 + 31 <= p_first && key0 >= lo_last);
 #pragma unroll
         for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, masked);
       }
@@ -284,7 +288,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
-    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink) {
+    float scale, int q_blocks, const float* __restrict__ slopes, int has_sink, float sink, int keep_first) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
   constexpr int NT = CK / 32;             // score tiles of a chunk of CK keys
@@ -311,7 +315,10 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int* bt = block_table + (long)(seq_rows ? __builtin_amdgcn_readfirstlane(seq_rows[b]) : b) * table_stride;
   const int blk_first = before + qb * QB, blk_last = before + min(qb * QB + QB - 1, q_len - 1);
   const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
-  const int ck0 = blk_lo / CK, ck1 = blk_last / CK;
+  // (kept first keys: as in the kernel above, their chunks before the window's first chunk are numbered in front of it)
+  const int ckw = blk_lo / CK, ck1 = blk_last / CK;
+  const int ck0 = ckw - (BIAS ? min((keep_first + CK - 1) / CK, ckw) : 0);
+  auto real = [&](int ck) { return (BIAS && ck < ckw) ? ck - ck0 : ck; };
   const int qi0 = qb * QB + wave * 32;
   const bool active = qi0 < q_len;
   const bool q_ok = qi0 + n < q_len;
@@ -412,7 +419,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int key = key0 + 32 * t + 16 * (v >> 3) + 8 * h + (v & 7);
-          s[t][v] = (key >= lo_mine && key <= p_mine) ? s[t][v] : -INFINITY;
+          s[t][v] = ((key >= lo_mine || (BIAS && key < keep_first)) && key <= p_mine) ? s[t][v] : -INFINITY;
         }
     }
     float mx = s[0][0];
@@ -458,7 +465,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   };
 
 #pragma unroll
-  for (int r = 0; r < AHEAD; ++r) fetch(min(ck0 + r, ck1), rk[r], rv[r]);
+  for (int r = 0; r < AHEAD; ++r) fetch(real(min(ck0 + r, ck1)), rk[r], rv[r]);
   stage(0, rk[0], rv[0]);
   __syncthreads();
   int buf = 0;
@@ -467,14 +474,14 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     for (int r = 0; r < AHEAD; ++r) {
       const int ck = base + r;
       if (ck > ck1) break;
-      const int key0 = ck * CK;
+      const int key0 = real(ck) * CK;
       // the registers of this chunk are free (it lies in shared memory): ask for the chunk AHEAD further;
       // unconditional (the last chunk again at the end): a branch around the loads makes the compiler
       // wait for all of them at once
-      fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);
-      if (ck >= ck_first && ck <= ck_last) {
+      fetch(real(min(ck + AHEAD, ck1)), rk[r], rv[r]);
+      if (active && (ck >= ck_first || (BIAS && key0 < keep_first)) && ck <= ck_last) {
         // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
-        chunk(buf, key0, !(key0 + CK - 1 <= p_first && key0 >= lo_last));
+        chunk(buf, key0, (BIAS && ck < ckw) || !(key0 + CK - 1 <= p_first && key0 >= lo_last));
       }
       if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
       __syncthreads();
@@ -521,7 +528,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
                                      const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
                                      int max_q_len, int n_heads, int n_kv, int head_dim, int page_size, int window,
                                      float scale, int wide_from, const float* slopes, int has_sink, float sink,
-                                     hipStream_t stream) {
+                                     int keep_first, hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && cu_seqlens && kv_before && block_table && out,
               "gl3_attention_prefill: null argument");
@@ -543,11 +550,12 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   GL3_REQUIRE(n_seqs <= 65535 && q_blocks <= 65535, "gl3_attention_prefill: %d sequences / %d blocks of queries exceed the grid",
               n_seqs, q_blocks);
   dim3 grid((unsigned)z, n_seqs, q_blocks), block(256);
-  const bool biased = slopes != nullptr || has_sink;
+  GL3_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "gl3_attention_prefill: %d kept first keys without a window", keep_first);
+  const bool biased = slopes != nullptr || has_sink || keep_first > 0;    // (the kernels that know of kept first keys)
   if (wide) {
 #define PF_ARGS                                                                                                     \
   (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table,     \
-      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks, slopes, has_sink, sink, keep_first
 #define GOW(HS, CK, AH, OCC)                                                                                        \
   do {                                                                                                              \
     if (biased) attention_prefill_wide_kernel<HS, CK, AH, OCC, true><<<grid, block, 0, stream>>>(PF_ARGS);          \

@@ -464,10 +464,7 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     disabled = _off(ctx)
     extras = dict(slopes=slopes, sink=sink)
-    keep_first = int(keep_first or 0) if window else 0
-    if keep_first:
-        return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
-                                   head_dim, page, window, scale, v_head_dim=v_head_dim, keep_first=keep_first, **extras)
+    extras["keep_first"] = int(keep_first or 0) if window else 0
     if q.dtype == torch.bfloat16 and (v_head_dim is None or v_head_dim == head_dim):     # (the matrix-core kernels: values of the keys' size)
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):

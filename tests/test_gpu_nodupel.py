@@ -60,13 +60,16 @@ def attention_on_gpu(q, k, v, positions, dtype, window, keep, scale, page=64, ke
     if kernel == "generic":
         K.attention_generic(qd, kc, vc, i32(positions), i32([0] * T), table, out, H, G, D, page, window, scale,
                             v_head_dim=Dv, keep_first=keep)
-    elif kernel == "decode":
-        K.attention_decode(qd, kc, vc, i32(positions), i32([0] * T), table, out, H, G, D, page, window, scale, 1, None, None,
-                           keep_first=keep)
+    elif kernel[0] == "decode":
+        n = kernel[1]
+        part_o = torch.zeros((T, H, n, D), dtype=torch.float32, device=DEV) if n > 1 else None
+        part_ml = torch.zeros((T, H, n, 2), dtype=torch.float32, device=DEV) if n > 1 else None
+        K.attention_decode(qd, kc, vc, i32(positions), i32([0] * T), table, out, H, G, D, page, window, scale, n, part_o,
+                           part_ml, keep_first=keep)
     else:
         # the tokens of one sequence, the first of them at positions[0]
         K.attention_prefill(qd, kc, vc, i32([0, T]), i32([positions[0]]), table, out, T, H, G, D, page, window, scale,
-                            keep_first=keep)
+                            wide_from=kernel[1], keep_first=keep)
     return out.float().cpu().numpy().reshape(T, H, Dv)
 
 
@@ -108,6 +111,42 @@ def test_kept_first_keys_and_the_window_edges(dtype, H, G, D, Dv, window, keep):
         np.testing.assert_allclose(got, ref, atol=2e-4 if dtype == "float32" else 0.25, err_msg=f"marked {marked}")
         for t, see in enumerate(sees):      # the marked value dominates exactly where the key is visible
             assert (np.abs(got[t]).mean() > 10.0) == see, (marked, positions[t])
+
+
+MATRIX_CORE_CASES = [(8, 1, 64, 37, 5), (4, 2, 32, 64, 33), (2, 2, 96, 20, 70), (3, 1, 128, 130, 64), (4, 4, 64, 100, 0)]
+
+
+@pytest.mark.parametrize("splits", [1, 3])
+@pytest.mark.parametrize("H, G, D, window, keep", MATRIX_CORE_CASES)
+def test_decode_attention_on_the_matrix_cores_keeps_the_first_keys(H, G, D, window, keep, splits):
+    rng = np.random.default_rng([H, D, window, keep, splits])
+    S = 330
+    for marked in (max(keep - 1, 0), keep, 200 - window, 200 - window + 1, 64):
+        q, k, v = marked_case(H, G, D, D, S, marked, rng)
+        positions = sorted({p for p in (marked, marked + 1, marked + window - 1, marked + window, marked + window + 1, 63,
+                                        64, 65, 127, 128, 199, 200, 201, 329) if marked <= p < S} | {0, 1, keep, keep + 1, max(0, marked - 1)})
+        ref = plain_attention_at(q[positions], k, v, positions, window, keep, 0.25)
+        got = attention_on_gpu(q[positions], k, v, positions, "bfloat16", window, keep, 0.25, kernel=("decode", splits))
+        np.testing.assert_allclose(got, ref, atol=0.25, err_msg=f"marked {marked}")
+        for t, p in enumerate(positions):
+            assert (np.abs(got[t]).mean() > 10.0) == P.visible(p, marked, window, keep), (marked, p)
+
+
+@pytest.mark.parametrize("wide_from", [1, 10 ** 6])
+@pytest.mark.parametrize("H, G, D, window, keep", MATRIX_CORE_CASES)
+def test_prompt_attention_on_the_matrix_cores_keeps_the_first_keys(H, G, D, window, keep, wide_from):
+    """Both prompt kernels, a prompt from its start and a portion that follows 150 cached tokens."""
+    rng = np.random.default_rng([H, D, window, keep, 77])
+    S = 330
+    for marked in (max(keep - 1, 0), keep, 200 - window, 64):
+        for first in (0, 150):
+            q, k, v = marked_case(H, G, D, D, S, marked, rng)
+            positions = list(range(first, S))
+            ref = plain_attention_at(q[positions], k, v, positions, window, keep, 0.25)
+            got = attention_on_gpu(q[positions], k, v, positions, "bfloat16", window, keep, 0.25, kernel=("prompt", wide_from))
+            np.testing.assert_allclose(got, ref, atol=0.25, err_msg=f"marked {marked}, from {first}")
+            for t, p in enumerate(positions):
+                assert (np.abs(got[t]).mean() > 10.0) == P.visible(p, marked, window, keep), (marked, first, p)
 
 
 # ----------------------------------------------------------------- rotations of heads, the gate per head
