@@ -23,6 +23,9 @@ machine: a Melizen model (windowed attention with a distance bias and a sink in 
 rule in the others, one norm a layer, a bounded gated feed-forward) with the width, feed-forward size, head sizes,
 vocabulary and layer count of ``--shape`` (``--layers`` for fewer), random weights. Its line carries prefill and
 decode throughput of both and their ratio; the default run and its line are not touched by it.
+``--arch nodupel`` does the same for a Nodupel model (every fourth layer a minGRU, the others an attention with
+rotated values, a gate per head and a window that keeps the first keys beside a time mixing with heads of 64; the
+shape's gated feed-forward in every layer; a hashed table of token pairs beside the embedding; no loop).
 """
 import argparse
 import json
@@ -107,8 +110,9 @@ def main():
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
-    ap.add_argument("--arch", default="llama", choices=["llama", "melizen"],
-                    help="melizen: a Melizen model of the shape's sizes beside Llama layers of equal size (a line of its own form)")
+    ap.add_argument("--arch", default="llama", choices=["llama", "melizen", "nodupel"],
+                    help="melizen, nodupel: a model of that design with the shape's sizes beside Llama layers of equal size "
+                         "(a line of its own form)")
     ap.add_argument("--without", default="", help="names of fast paths to switch off for a comparison on the same machine, "
                     "comma-separated (parts/ops.py: tiled, packed, fused, wide, ...); the line then says so in `config`")
     args = ap.parse_args()
@@ -120,8 +124,8 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
 
-    if args.arch == "melizen":
-        return melizen_beside_llama(args)
+    if args.arch in ("melizen", "nodupel"):
+        return other_beside_llama(args)
 
     import numpy as np
     import torch
@@ -325,9 +329,26 @@ def melizen_config(shape, layers, window=1024):
             "norm": {"eps": 1e-5}, "layers": [attn if i % 2 == 0 else delta for i in range(layers)]}
 
 
-def melizen_beside_llama(args):
-    """Prefill of one prompt and decode steps at --batch for a Melizen model and for Llama layers of equal size,
-    one after the other on the same machine."""
+def nodupel_config(shape, layers, window=1024, keep_first=4):
+    """A Nodupel model with the sizes of a Llama shape: every fourth layer a minGRU of the model's width, the others an
+    attention with the shape's heads (rotated values, a gate per head, a window that keeps the first keys) beside a
+    time mixing with heads of 64 over the model's width; the shape's feed-forward in every layer; no loop."""
+    d, F = shape["hidden_size"], shape["intermediate_size"]
+    H, G, hs = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    mlp = {"kind": "dense", "ff": F}
+    left = {"heads": H, "kv_heads": G, "dim": hs, "vdim": hs, "scale": hs ** -0.5,
+            "rot": {"base": shape.get("rope_theta", 500000.0), "dims": hs}, "mask": {"size": window, "keep_first": keep_first}}
+    side = {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": {"heads": d // 64, "dim": 64}}}
+    gru = {"type": "mingru", "mlp": mlp, "mixer": {"width": d}}
+    return {"architecture": "Nodupel", "vocab": shape["vocab_size"], "width": d, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "logit_softcap": 30.0, "max_positions": shape["max_position_embeddings"], "decay_rank": [64] * layers,
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+            "layers": [gru if i % 4 == 0 else side for i in range(layers)]}
+
+
+def other_beside_llama(args):
+    """Prefill of one prompt and decode steps at --batch for a model of another design (--arch) and for Llama layers
+    of equal size, one after the other on the same machine."""
     import numpy as np
     import torch
     import gpullama3_java_amd as g
@@ -339,7 +360,9 @@ def melizen_beside_llama(args):
     prompt_len, prefill_len = args.prompt_len, args.prefill_len
     per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
-    configs = {"melizen": g.config_from_dict(melizen_config(shape, layers)),
+    arch = args.arch
+    make = {"melizen": melizen_config, "nodupel": nodupel_config}[arch]
+    configs = {arch: g.config_from_dict(make(shape, layers)),
                "llama": g.config_from_dict({**shape, "num_hidden_layers": layers})}
     results = {}
     for name, cfg in configs.items():
@@ -389,18 +412,19 @@ def melizen_beside_llama(args):
               file=sys.stderr, flush=True)
         del eng
         torch.cuda.empty_cache()
-    m, l = results["melizen"], results["llama"]
+    m, l = results[arch], results["llama"]
+    title = arch.capitalize()
     line = {
-        "metric": f"decode tok/s at batch {B}, Melizen model of the {shape_name}'s sizes ({prompt_len}-token prompts)",
+        "metric": f"decode tok/s at batch {B}, {title} model of the {shape_name}'s sizes ({prompt_len}-token prompts)",
         "value": m["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": m["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic: random N(0,0.02) weights, uniform random token ids",
-        "config": {"model": f"Melizen, sizes of the {shape_name}", "layers": layers, "global_batch": B,
+        "config": {"model": f"{title}, sizes of the {shape_name}", "layers": layers, "global_batch": B,
                    "seq_len": shape["max_position_embeddings"], "prompt_len": prompt_len, "prefill_len": prefill_len,
                    "attention_window": 1024, "parallelism": "single GPU", "sampling": "greedy on device",
                    **({"without": args.without} if args.without else {})},
-        "melizen": m, "llama_of_equal_size": l,
-        "melizen_over_llama": {"prefill_time": round(m["prefill_ms"] / l["prefill_ms"], 3),
+        arch: m, "llama_of_equal_size": l,
+        f"{arch}_over_llama": {"prefill_time": round(m["prefill_ms"] / l["prefill_ms"], 3),
                                "decode_step_time": round(m["decode_ms_per_step"] / l["decode_ms_per_step"], 3)},
     }
     print(json.dumps(line))

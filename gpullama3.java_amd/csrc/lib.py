@@ -61,9 +61,9 @@ def _declare(lib):
         "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
         "gl3_concat_rows": [P, P, P, I, I, I, P],
         "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P],
-        "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P],
+        "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, P, I, L, P],
-        "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, P],
+        "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
         "gl3_shift_mix": [P, I, I, P, I, P, L, P, P, P, P, I, I, I, P],
         "gl3_timemix": [P, P, P, P, P, P, L, L, P, P, P, I, I, I, P],
         "gl3_head_norm_gate": [P, P, P, F, P, I, I, I, I, P],
@@ -510,8 +510,10 @@ def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, g
            "rotate_heads")
 
 
-def sides_norm_add(x, a, b, wa, wb, eps, factor):
-    """x += factor * (a / rms(a) * wa + b / rms(b) * wb); all float32, a and b [T, d] like x (b may be None)."""
+def sides_norm_add(x, a, b, wa, wb, eps, factor, ssq=None, next_weight=None, xg=None):
+    """x += factor * (a / rms(a) * wa + b / rms(b) * wb); all float32, a and b [T, d] like x (b may be None).
+    ``ssq`` (at least 64 floats, at most 64 tokens) receives each completed row's sum of squares; with it ``xg`` [T, d]
+    bfloat16 may receive ``next_weight * row``, the rows as the product after the next norm reads them."""
     _dev(x, "x", torch.float32); _dev(a, "a", torch.float32); _dev(wa, "wa", torch.float32)
     if x.dim() != 2 or a.shape != x.shape or wa.shape != (x.shape[1],):
         raise KernelError(f"sides_norm_add: x {tuple(x.shape)}, a {tuple(a.shape)}, weight {tuple(wa.shape)}")
@@ -519,8 +521,16 @@ def sides_norm_add(x, a, b, wa, wb, eps, factor):
         _dev(b, "b", torch.float32); _dev(wb, "wb", torch.float32)
         if b.shape != x.shape or wb.shape != wa.shape:
             raise KernelError(f"sides_norm_add: b {tuple(b.shape)}, weight {tuple(wb.shape)}")
+    if ssq is not None:
+        _dev(ssq, "ssq", torch.float32)
+        if ssq.numel() < 64 or x.shape[0] > 64:
+            raise KernelError("sides_norm_add: sums of squares need 64 floats and at most 64 tokens")
+    _check_next(next_weight, xg, x.shape[0], x.shape[1], "sides_norm_add")
+    if xg is not None and (ssq is None or not xg.is_contiguous()):
+        raise KernelError("sides_norm_add: the next norm's rows come with the sums of squares, contiguous")
     _check(library().gl3_sides_norm_add(_ptr(x), _ptr(a), _ptr(b), _ptr(wa), _ptr(wb) if b is not None else c_void_p(0),
-                                        float(eps), float(factor), x.shape[0], x.shape[1], _stream()), "sides_norm_add")
+                                        float(eps), float(factor), x.shape[0], x.shape[1], _ptr(ssq), _ptr(next_weight),
+                                        _ptr(xg), _stream()), "sides_norm_add")
 
 
 def tanh_rows(src, out):
@@ -531,18 +541,28 @@ def tanh_rows(src, out):
     _check(library().gl3_tanh_rows(_ptr(src), _ptr(out), _code(out, "out"), src.numel(), _stream()), "tanh_rows")
 
 
-def mingru_scan(proj, width, state, cu_seqlens, slot_ids, out):
+MINGRU_RUN = 32      # tokens of a run of the three-pass scan (MG_RUN in mixers.hip)
+
+
+def mingru_scan(proj, width, state, cu_seqlens, slot_ids, out, max_q_len=1, runs=None):
     """The minGRU recurrence over the step's tokens from the state in each sequence's slot: ``proj`` [T, >= 3 width]
     float32 holds the update gate's, the candidate's and the output gate's sums; ``out`` [T, width] receives
-    S_t * silu(gate); ``state`` [slots, >= width] float32 is advanced."""
+    S_t * silu(gate); ``state`` [slots, >= width] float32 is advanced. With ``runs`` (float32, at least
+    2 * sequences * ceil(max_q_len / 32) * width elements) and a longest sequence of ``max_q_len`` > 32 tokens the scan
+    runs in three passes over runs of 32 tokens."""
     _dev(proj, "proj", torch.float32, contiguous=False); _dev(state, "state", torch.float32, contiguous=False); _dev(out, "out")
     _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
     T, B = proj.shape[0], slot_ids.numel()
     if (state.dim() != 2 or state.stride(1) != 1 or proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < 3 * width or out.shape != (T, width) or state.dim() != 2
             or state.shape[1] < width or cu_seqlens.numel() != B + 1):
         raise KernelError(f"mingru_scan: proj {tuple(proj.shape)}, out {tuple(out.shape)}, state {tuple(state.shape)}")
+    if runs is not None:
+        _dev(runs, "runs", torch.float32)
+        if runs.numel() < 2 * B * -(-int(max_q_len) // MINGRU_RUN) * width:
+            raise KernelError(f"mingru_scan: scratch of {runs.numel()} floats for {B} sequences of up to {max_q_len} tokens")
     _check(library().gl3_mingru_scan(_ptr(proj), proj.stride(0), int(width), _ptr(state), state.stride(0), _ptr(cu_seqlens),
-                                     _ptr(slot_ids), _ptr(out), _code(out, "out"), B, _stream()), "mingru_scan")
+                                     _ptr(slot_ids), _ptr(out), _code(out, "out"), B, int(max_q_len), _ptr(runs), _stream()),
+           "mingru_scan")
 
 
 def shift_mix(h, mu, state, cu_seqlens, seq_of_token, slot_ids, out, one_token_each=False):
@@ -565,8 +585,8 @@ def shift_mix(h, mu, state, cu_seqlens, seq_of_token, slot_ids, out, one_token_e
 
 def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, H, D):
     """The decayed matrix per head, token by token from the state in each sequence's slot (``mixers.hip``): r, k, v,
-    w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D]; ``out`` [T, H D] float32 receives the raw
-    read-outs; ``state`` [slots, >= state_off + H D D] float32."""
+    w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D]; ``out``
+    [T, H D] float32 receives the raw read-outs; ``state`` [slots, >= state_off + H D D] float32."""
     for t, n in ((r, "r"), (k, "k"), (v, "v"), (w_log, "w_log"), (bonus, "bonus"), (out, "out")):
         _dev(t, n, torch.float32)
     _dev(state, "state", torch.float32, contiguous=False)

@@ -142,16 +142,20 @@ extern "C" int gl3_rotate_heads(void* rows, int dtype, long ld, const int* posit
 }
 
 // ----------------------------------------------------------------- x += f * (a / rms(a) * wa + b / rms(b) * wb)
-// One block a token. `b` may be null (one side only). Sums in an order that depends on d alone.
-__global__ __launch_bounds__(256) void sides_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a,
-                                                              const float* __restrict__ b, const float* __restrict__ wa,
-                                                              const float* __restrict__ wb, float eps, float f, int d) {
+// One block a token. `b` may be null (one side only). Sums in an order that depends on d and the block's size alone.
+// ssq (may be null; then at most 64 tokens): ssq[t] = the sum of squares of the completed row, for a norm that is
+// folded into the product that follows; with it next_weight [d] and xg [T][d]: xg = bfloat16(next_weight * row).
+__global__ __launch_bounds__(1024) void sides_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a,
+                                                               const float* __restrict__ b, const float* __restrict__ wa,
+                                                               const float* __restrict__ wb, float eps, float f, int d,
+                                                               float* __restrict__ ssq, const float* __restrict__ next_weight,
+                                                               bf16_t* __restrict__ xg) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const float* pa = a + t * d;
   const float* pb = b ? b + t * d : nullptr;
   float sa = 0.f, sb = 0.f;
-  for (int i = threadIdx.x; i < d; i += 256) {
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
     const float va = pa[i];
     sa += va * va;
     if (pb) {
@@ -162,18 +166,31 @@ __global__ __launch_bounds__(256) void sides_norm_add_kernel(float* __restrict__
   sa = block_sum(sa, scratch);
   sb = block_sum(sb, scratch);
   const float ia = 1.0f / sqrtf(sa / (float)d + eps), ib = 1.0f / sqrtf(sb / (float)d + eps);
-  for (int i = threadIdx.x; i < d; i += 256) {
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = pa[i] * ia * wa[i];
     if (pb) v += pb[i] * ib * wb[i];
-    x[t * d + i] += f * v;
+    const float xn = x[t * d + i] + f * v;
+    x[t * d + i] = xn;
+    ss += xn * xn;
+    if (xg) xg[t * d + i] = static_cast<bf16_t>(next_weight[i] * xn);
+  }
+  if (ssq) {
+    ss = block_sum(ss, scratch);
+    if (threadIdx.x == 0) ssq[t] = ss;
   }
 }
 
 extern "C" int gl3_sides_norm_add(float* x, const float* a, const float* b, const float* wa, const float* wb, float eps,
-                                  float f, int n_tokens, int d, hipStream_t stream) {
+                                  float f, int n_tokens, int d, float* ssq, const float* next_weight, void* xg,
+                                  hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(x && a && wa && (!b || wb) && n_tokens > 0 && d > 0, "gl3_sides_norm_add: bad arguments");
-  sides_norm_add_kernel<<<dim3(n_tokens), dim3(256), 0, stream>>>(x, a, b, wa, wb, eps, f, d);
+  GL3_REQUIRE(!ssq || n_tokens <= 64, "gl3_sides_norm_add: sums of squares are kept for at most 64 rows");
+  GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || ssq),
+              "gl3_sides_norm_add: the next norm's weight and its rows come together, with the sums of squares");
+  const int threads = d >= 1024 ? 1024 : ((d + 63) / 64) * 64;
+  sides_norm_add_kernel<<<dim3(n_tokens), dim3(threads), 0, stream>>>(x, a, b, wa, wb, eps, f, d, ssq, next_weight, (bf16_t*)xg);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -225,17 +242,105 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const float* __restric
   *held = S;
 }
 
+// The same recurrence for long prompts, in three passes over runs of MG_RUN tokens. S_t = (1 - z_t) S_(t-1) + z_t c_t
+// is linear in S, so a run of tokens maps the state before it to A S + B with A = prod (1 - z), B = the run's scan
+// from zero: (1) every run's A and B, all runs at once; (2) per sequence and channel the state in front of every run,
+// run after run (a prompt of 2,048 tokens: 64 steps, not 2,048), and the sequence's last state into its slot; (3)
+// every run again from its own start, writing the outputs. Twice the arithmetic, a thirtieth of the chain.
+#define MG_RUN 32
+
+__global__ __launch_bounds__(256) void mingru_runs_kernel(const float* __restrict__ proj, long ld, int W,
+                                                           const int* __restrict__ cu_seqlens, float* __restrict__ run_a,
+                                                           float* __restrict__ run_b, int n_runs) {
+  const int c = blockIdx.x * 256 + threadIdx.x, run = blockIdx.y, seq = blockIdx.z;
+  const int t0 = cu_seqlens[seq] + run * MG_RUN, end = cu_seqlens[seq + 1];
+  if (c >= W || t0 >= end) return;
+  const int t1 = t0 + MG_RUN < end ? t0 + MG_RUN : end;
+  float A = 1.f, B = 0.f;
+#pragma unroll 4
+  for (int t = t0; t < t1; ++t) {
+    const float* p = proj + (long)t * ld + c;
+    const float pz = p[0], pu = p[W];
+    const float z = 1.0f / (1.0f + expf(-pz));
+    const float cand = pu >= 0.f ? pu + 0.5f : 1.0f / (1.0f + expf(-pu));
+    A *= 1.0f - z;
+    B = (1.0f - z) * B + z * cand;
+  }
+  const long at = ((long)seq * n_runs + run) * W + c;
+  run_a[at] = A;
+  run_b[at] = B;
+}
+
+// run_a: in A, out the state in front of the run
+__global__ __launch_bounds__(256) void mingru_carry_kernel(float* __restrict__ run_a, const float* __restrict__ run_b,
+                                                            float* __restrict__ state, long state_stride,
+                                                            const int* __restrict__ cu_seqlens,
+                                                            const int* __restrict__ slot_ids, int W, int n_runs) {
+  const int c = blockIdx.x * 256 + threadIdx.x, seq = blockIdx.y;
+  if (c >= W) return;
+  float* held = state + (long)slot_ids[seq] * state_stride + c;
+  float S = *held;
+  const int n = (cu_seqlens[seq + 1] - cu_seqlens[seq] + MG_RUN - 1) / MG_RUN;
+  for (int run = 0; run < n; ++run) {
+    const long at = ((long)seq * n_runs + run) * W + c;
+    const float A = run_a[at], B = run_b[at];
+    run_a[at] = S;
+    S = A * S + B;
+  }
+  *held = S;
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void mingru_apply_kernel(const float* __restrict__ proj, long ld, int W,
+                                                            const int* __restrict__ cu_seqlens,
+                                                            const float* __restrict__ run_start, int n_runs,
+                                                            TO* __restrict__ out) {
+  const int c = blockIdx.x * 256 + threadIdx.x, run = blockIdx.y, seq = blockIdx.z;
+  const int t0 = cu_seqlens[seq] + run * MG_RUN, end = cu_seqlens[seq + 1];
+  if (c >= W || t0 >= end) return;
+  const int t1 = t0 + MG_RUN < end ? t0 + MG_RUN : end;
+  float S = run_start[((long)seq * n_runs + run) * W + c];
+#pragma unroll 4
+  for (int t = t0; t < t1; ++t) {
+    const float* p = proj + (long)t * ld + c;
+    const float pz = p[0], pu = p[W], pg = p[2 * W];
+    const float z = 1.0f / (1.0f + expf(-pz));
+    const float cand = pu >= 0.f ? pu + 0.5f : 1.0f / (1.0f + expf(-pu));
+    S = (1.0f - z) * S + z * cand;
+    out[(long)t * W + c] = from_f32<TO>(S * (pg / (1.0f + expf(-pg))));
+  }
+}
+
+// max_q_len: the most tokens a sequence brings (host's knowledge); runs [2][n_seqs][ceil(max_q_len / 32)][W] floats of
+// scratch (may be null: one pass, token by token).
 extern "C" int gl3_mingru_scan(const float* proj, long ld, int W, float* state, long state_stride, const int* cu_seqlens,
-                               const int* slot_ids, void* out, int out_dtype, int n_seqs, hipStream_t stream) {
+                               const int* slot_ids, void* out, int out_dtype, int n_seqs, int max_q_len, float* runs,
+                               hipStream_t stream) {
   if (n_seqs == 0) return 0;
   GL3_REQUIRE(proj && state && cu_seqlens && slot_ids && out && W > 0 && ld >= 3L * W && state_stride >= W &&
                   n_seqs > 0 && n_seqs <= 65535, "gl3_mingru_scan: bad arguments (W=%d ld=%ld B=%d)", W, ld, n_seqs);
+  GL3_REQUIRE(out_dtype == GL3_F32 || out_dtype == GL3_BF16, "gl3_mingru_scan: unknown dtype %d", out_dtype);
+  if (runs && max_q_len > MG_RUN) {
+    const int n_runs = (max_q_len + MG_RUN - 1) / MG_RUN;
+    GL3_REQUIRE(n_runs <= 65535, "gl3_mingru_scan: %d tokens a sequence exceed the grid", max_q_len);
+    float* run_a = runs;
+    float* run_b = runs + (long)n_seqs * n_runs * W;
+    dim3 grid((W + 255) / 256, n_runs, n_seqs), block(256);
+    mingru_runs_kernel<<<grid, block, 0, stream>>>(proj, ld, W, cu_seqlens, run_a, run_b, n_runs);
+    mingru_carry_kernel<<<dim3((W + 255) / 256, n_seqs), block, 0, stream>>>(run_a, run_b, state, state_stride, cu_seqlens,
+                                                                           slot_ids, W, n_runs);
+    if (out_dtype == GL3_F32)
+      mingru_apply_kernel<float><<<grid, block, 0, stream>>>(proj, ld, W, cu_seqlens, run_a, n_runs, (float*)out);
+    else
+      mingru_apply_kernel<bf16_t><<<grid, block, 0, stream>>>(proj, ld, W, cu_seqlens, run_a, n_runs, (bf16_t*)out);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((W + 255) / 256, n_seqs), block(256);
   if (out_dtype == GL3_F32)
     mingru_scan_kernel<float><<<grid, block, 0, stream>>>(proj, ld, W, state, state_stride, cu_seqlens, slot_ids, (float*)out);
-  else if (out_dtype == GL3_BF16)
+  else
     mingru_scan_kernel<bf16_t><<<grid, block, 0, stream>>>(proj, ld, W, state, state_stride, cu_seqlens, slot_ids, (bf16_t*)out);
-  else GL3_REQUIRE(false, "gl3_mingru_scan: unknown dtype %d", out_dtype);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -256,7 +361,8 @@ __global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ h,
   const int seq = seq_of_token[t];
   const bool from_step = t > cu_seqlens[seq];
   float* held = state + (long)slot_ids[seq] * state_stride;
-  for (int i = threadIdx.x; i < d; i += 256) {
+  // (grid y: the row's elements in runs of 256, one a thread: nothing in a thread waits for an earlier trip to memory)
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < d; i += 256 * gridDim.y) {
     const float cur = to_f32<T>(h[t * d + i]);
     const float prev = from_step ? to_f32<T>(h[(t - 1) * d + i]) : held[i];
     const float diff = prev - cur;
@@ -281,14 +387,14 @@ extern "C" int gl3_shift_mix(const void* h, int dtype, int d, const float* mu, i
                              int n_seqs, int one_token_each, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(h && mu && state && cu_seqlens && seq_of_token && slot_ids && out && d > 0 && n_mix > 0 && n_tokens > 0 &&
-                  n_seqs > 0 && state_stride >= d, "gl3_shift_mix: bad arguments");
+                  n_seqs > 0 && state_stride >= d && (d + 255) / 256 <= 65535, "gl3_shift_mix: bad arguments");
   const int inl = one_token_each && n_tokens == n_seqs;
   if (dtype == GL3_F32) {
-    shift_mix_kernel<float><<<dim3(n_tokens), dim3(256), 0, stream>>>((const float*)h, d, mu, n_mix, state, state_stride,
+    shift_mix_kernel<float><<<dim3(n_tokens, (d + 255) / 256), dim3(256), 0, stream>>>((const float*)h, d, mu, n_mix, state, state_stride,
                                                                       cu_seqlens, seq_of_token, slot_ids, (float*)out, n_tokens, inl);
     if (!inl) keep_last_rows_kernel<float><<<dim3(n_seqs), dim3(256), 0, stream>>>((const float*)h, d, state, state_stride, cu_seqlens, slot_ids);
   } else if (dtype == GL3_BF16) {
-    shift_mix_kernel<bf16_t><<<dim3(n_tokens), dim3(256), 0, stream>>>((const bf16_t*)h, d, mu, n_mix, state, state_stride,
+    shift_mix_kernel<bf16_t><<<dim3(n_tokens, (d + 255) / 256), dim3(256), 0, stream>>>((const bf16_t*)h, d, mu, n_mix, state, state_stride,
                                                                        cu_seqlens, seq_of_token, slot_ids, (bf16_t*)out, n_tokens, inl);
     if (!inl) keep_last_rows_kernel<bf16_t><<<dim3(n_seqs), dim3(256), 0, stream>>>((const bf16_t*)h, d, state, state_stride, cu_seqlens, slot_ids);
   } else GL3_REQUIRE(false, "gl3_shift_mix: unknown dtype %d", dtype);
@@ -300,11 +406,17 @@ extern "C" int gl3_shift_mix(const void* h, int dtype, int d, const float* mu, i
 // Per sequence and head a matrix S [D keys][D values] in 32-bit (state: [H][D][D] floats from `state_off` of the
 // slot's row). r, k, v, wl are [T][H*D] float; the decay of key channel i is w = exp(-exp(wl)); bonus [H][D].
 //   o_t[j] = sum_i r_t[i] (S[i][j] + bonus[i] k_t[i] v_t[j]);   S[i][j] <- w_t[i] S[i][j] + k_t[i] v_t[j]
-// grid (H, sequences). A thread owns RP rows of one column j in registers (D * ceil(D / RP) threads a block); a
-// token's r, k, w, v reach the block through shared memory four tokens at a time, the parts of a column's sum are
-// added in shared memory in the order of the parts. Tokens are walked in order from the state in the slot.
-#define TM_CH 4
+// Tokens are walked in order from the state in the slot, so every cut of a sequence into steps gives the same sums.
+//
+// grid (H, sequences). A wave owns RP rows (keys) of 64 columns (values): a lane keeps its column's RP elements of S
+// in registers. A round of `ch` tokens' r, k, w (the two exponentials are taken here, once an element) and v reaches
+// the block through shared memory: every thread loads its share of the NEXT round into registers before it works on
+// the current one, and stores it afterwards, so a trip to memory is paid once a round and hidden behind the work.
+// The waves' parts of a column's sum over the rows meet in shared memory too, and are added in the order of the
+// parts after the round's one barrier. Both areas have two buffers, which is why one barrier a round is enough: a
+// wave writes a buffer again only after the barrier that every wave passes after its last read of it.
 #define TM_MAXD 256
+#define TM_LD 8           // loads a thread has on their way for the next round
 
 template <int RP>
 __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__ r, const float* __restrict__ k,
@@ -313,63 +425,101 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
                                                         long state_stride, long state_off,
                                                         const int* __restrict__ cu_seqlens,
                                                         const int* __restrict__ slot_ids, float* __restrict__ o, int H,
-                                                        int D) {
-  __shared__ float sr[TM_CH][TM_MAXD], sk[TM_CH][TM_MAXD], sw[TM_CH][TM_MAXD], sv[TM_CH][TM_MAXD];
-  __shared__ float parts[TM_CH][1024];
-  __shared__ float su[TM_MAXD];
+                                                        int D, int ch) {
+  extern __shared__ __attribute__((aligned(16))) float tm_shared[];
   const int head = blockIdx.x, seq = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
-  const int j = tid % D, part = tid / D, i0 = part * RP;
-  const int P = (D + RP - 1) / RP;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int CG = (D + 63) / 64;                // groups of 64 columns
+  const int P = (D + RP - 1) / RP;             // parts of RP rows
+  const int cols = CG * 64, Dr = P * RP;       // a staged row's length: whole parts
+  const int part = wave / CG, j = (wave - part * CG) * 64 + lane, i0 = part * RP;
+  const bool col_ok = j < D;
   const long HD = (long)H * D;
+  // shared memory: stage [2][ch][4][Dr] (r, k, w, v of a token), parts [2][ch][P * cols]
+  float* stage = tm_shared;
+  float* parts = tm_shared + 2 * ch * 4 * Dr;
   float* held = state + (long)slot_ids[seq] * state_stride + state_off + (long)head * D * D;
-  float S[RP];
+  float S[RP], ub[RP];
 #pragma unroll
   for (int ii = 0; ii < RP; ++ii) {
-    const int i = i0 + ii;
-    S[ii] = i < D ? held[(long)i * D + j] : 0.f;
+    S[ii] = (col_ok && i0 + ii < D) ? held[(long)(i0 + ii) * D + j] : 0.f;
+    ub[ii] = i0 + ii < D ? bonus[head * D + i0 + ii] : 0.f;
   }
-  for (int i = tid; i < D; i += nt) su[i] = bonus[head * D + i];
   const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
-  for (int tb = t0; tb < t1; tb += TM_CH) {
-    const int n = t1 - tb < TM_CH ? t1 - tb : TM_CH;
-    __syncthreads();
-    for (int idx = tid; idx < n * D; idx += nt) {
-      const int tt = idx / D, i = idx - tt * D;
-      const long at = (long)(tb + tt) * HD + head * D + i;
-      sr[tt][i] = r[at];
-      sk[tt][i] = k[at];
-      sv[tt][i] = v[at];
-      sw[tt][i] = expf(-expf(wl[at]));
+  float ld[TM_LD];
+  // item idx of a round: token idx / (4 D), array (idx / D) % 4, element idx % D
+  auto fetch = [&](int tb) {
+    const int n = t1 - tb < ch ? t1 - tb : ch;
+#pragma unroll
+    for (int m = 0; m < TM_LD; ++m) {
+      const int idx = tid + m * nt;
+      float x = 0.f;
+      if (idx < n * 4 * D) {
+        const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
+        const float* src = a == 0 ? r : a == 1 ? k : a == 2 ? wl : v;
+        x = src[(long)(tb + tt) * HD + (long)head * D + i];
+      }
+      ld[m] = x;
     }
-    __syncthreads();
+  };
+  auto put = [&](int buf, int tb) {
+    const int n = t1 - tb < ch ? t1 - tb : ch;
+#pragma unroll
+    for (int m = 0; m < TM_LD; ++m) {
+      const int idx = tid + m * nt;
+      if (idx < n * 4 * D) {
+        const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
+        stage[((buf * ch + tt) * 4 + a) * Dr + i] = a == 2 ? expf(-expf(ld[m])) : ld[m];
+      }
+    }
+  };
+  if (t0 < t1) {
+    fetch(t0);
+    put(0, t0);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t0; tb < t1; tb += ch, buf ^= 1) {
+    const int n = t1 - tb < ch ? t1 - tb : ch;
+    if (tb + ch < t1) fetch(tb + ch);
     for (int tt = 0; tt < n; ++tt) {
-      const float vj = sv[tt][j];
+      const float* row = stage + (buf * ch + tt) * 4 * Dr;
+      const float vj = col_ok ? row[3 * Dr + j] : 0.f;
       float acc = 0.f;
 #pragma unroll
-      for (int ii = 0; ii < RP; ++ii) {
-        const int i = i0 + ii;
-        if (i < D) {
-          const float kv = sk[tt][i] * vj;
-          acc = fmaf(sr[tt][i], S[ii] + su[i] * kv, acc);
-          S[ii] = sw[tt][i] * S[ii] + kv;
+      for (int i4 = 0; i4 < RP; i4 += 4) {
+        if (i0 + i4 < D) {     // (the same for the whole wave; rows behind D inside a group of four hold what was staged: nothing they add is read)
+          const float4 r4 = *(const float4*)(row + i0 + i4), k4 = *(const float4*)(row + Dr + i0 + i4),
+                       w4 = *(const float4*)(row + 2 * Dr + i0 + i4);
+          const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (i0 + i4 + e < D) {
+              const float kv = kk[e] * vj;
+              acc = fmaf(rr[e], fmaf(ub[i4 + e], kv, S[i4 + e]), acc);
+              S[i4 + e] = fmaf(ww[e], S[i4 + e], kv);
+            }
+          }
         }
       }
-      parts[tt][tid] = acc;
+      parts[(buf * ch + tt) * P * cols + part * cols + j] = acc;
     }
+    if (tb + ch < t1) put(buf ^ 1, tb + ch);
     __syncthreads();
     for (int idx = tid; idx < n * D; idx += nt) {
       const int tt = idx / D, jj = idx - tt * D;
       float sum = 0.f;
-      for (int p = 0; p < P; ++p) sum += parts[tt][p * D + jj];
-      o[(long)(tb + tt) * HD + head * D + jj] = sum;
+      for (int p = 0; p < P; ++p) sum += parts[(buf * ch + tt) * P * cols + p * cols + jj];
+      o[(long)(tb + tt) * HD + (long)head * D + jj] = sum;
     }
   }
 #pragma unroll
-  for (int ii = 0; ii < RP; ++ii) {
-    const int i = i0 + ii;
-    if (i < D) held[(long)i * D + j] = S[ii];
-  }
+  for (int ii = 0; ii < RP; ++ii)
+    if (col_ok && i0 + ii < D) held[(long)(i0 + ii) * D + j] = S[ii];
 }
+
+// rows a wave owns: 8 for heads of up to 64 (eight waves a head), 16 up to 128, 64 beyond
+static int timemix_rows(int D) { return D <= 64 ? 8 : D <= 128 ? 16 : 64; }
 
 extern "C" int gl3_timemix(const float* r, const float* k, const float* v, const float* wl, const float* bonus,
                            float* state, long state_stride, long state_off, const int* cu_seqlens, const int* slot_ids,
@@ -380,15 +530,20 @@ extern "C" int gl3_timemix(const float* r, const float* k, const float* v, const
   GL3_REQUIRE(D >= 1 && D <= TM_MAXD, "gl3_timemix: heads of %d elements: the kernel holds up to %d", D, TM_MAXD);
   GL3_REQUIRE(state_off >= 0 && state_off + (long)H * D * D <= state_stride, "gl3_timemix: the state's row of %ld floats", state_stride);
   dim3 grid(H, n_seqs);
-  if (D <= 128) {
-    const int P = (D + 15) / 16;
-    timemix_kernel<16><<<grid, dim3(D * P), 0, stream>>>(r, k, v, wl, bonus, state, state_stride, state_off, cu_seqlens,
-                                                        slot_ids, o, H, D);
-  } else {
-    const int P = (D + 63) / 64;
-    timemix_kernel<64><<<grid, dim3(D * P), 0, stream>>>(r, k, v, wl, bonus, state, state_stride, state_off, cu_seqlens,
-                                                        slot_ids, o, H, D);
-  }
+  const int RP = timemix_rows(D), CG = (D + 63) / 64, P = (D + RP - 1) / RP;
+  const int nt = 64 * CG * P, Dr = P * RP, per_token = 2 * 4 * Dr + 2 * P * CG * 64;
+  // tokens a round: what 60 KB of shared memory hold, what the threads' TM_LD loads each bring, 16 at most
+  int ch = 15360 / per_token;
+  if (ch > TM_LD * nt / (4 * D)) ch = TM_LD * nt / (4 * D);
+  if (ch > 16) ch = 16;
+  GL3_REQUIRE(ch >= 1 && nt <= 1024, "gl3_timemix: heads of %d do not fit the kernel's shared memory", D);
+  const size_t shared = (size_t)ch * per_token * sizeof(float);
+#define TM_GO(R) timemix_kernel<R><<<grid, dim3(nt), shared, stream>>>(r, k, v, wl, bonus, state, state_stride, state_off, \
+                                                                   cu_seqlens, slot_ids, o, H, D, ch)
+  if (RP == 8) TM_GO(8);
+  else if (RP == 16) TM_GO(16);
+  else TM_GO(64);
+#undef TM_GO
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -66,7 +66,10 @@ class MinGRU:
         proj = ctx.buffer("mingru_proj", (T, self.n_pad), torch.float32)
         ops.linear(h, self.w_in, proj, ops.EPI_STORE, ctx, bias=self.bias)
         y = ctx.buffer("mingru_out", (T, self.W), self.dtype)
-        K.mingru_scan(proj, self.W, ctx.slot_state(run.entry), ctx.cu_seqlens, ctx.slot_ids, y)
+        runs = None
+        if ctx.max_q_len > 2 * K.MINGRU_RUN:      # a long prompt: the scan in three passes over runs of tokens
+            runs = ctx.buffer("mingru_runs", (2, ctx.n_seqs, -(-ctx.max_q_len // K.MINGRU_RUN), self.W), torch.float32)
+        K.mingru_scan(proj, self.W, ctx.slot_state(run.entry), ctx.cu_seqlens, ctx.slot_ids, y, ctx.max_q_len, runs)
         ops.linear(y, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)
 
 

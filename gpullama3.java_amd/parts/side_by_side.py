@@ -87,6 +87,16 @@ class SideBySide:
             lo += size
         ctx.next_norm = next_norm
         ops.settle_residual(ctx, x)
+        if (getattr(ctx, "fuse", False) and T == ctx.n_tokens <= ops.FUSE_ROWS and "fused" not in ops._off(ctx)
+                and self.d % 16 == 0):
+            # the rows are complete after this kernel: it leaves what the norm that follows would use (the rows' sums of
+            # squares, and the rows times that norm's weight), so that the next product can take the norm over
+            norm, xg = ops._next_norm(ctx, self.d)
+            if norm is not None:
+                ssq = ctx.ssq_buffer(1)
+                K.sides_norm_add(x, outs[0], outs[1], self.w_left, self.w_right, self.spec.norm_eps, self.factor,
+                                 ssq, norm.weight_f32, xg)
+                return ops.residual_written(ctx, x, ssq, 1, xg, norm)
         K.sides_norm_add(x, outs[0], outs[1], self.w_left, self.w_right, self.spec.norm_eps, self.factor)
         ops.residual_written(ctx, x)
 

@@ -236,7 +236,11 @@ def test_mingru_scan_whole_and_in_pieces(W, dtype):
             live = [b for b in range(3) if hi[b] > lo[b]]
             rows = np.concatenate([proj[cu[b] + lo[b]:cu[b] + hi[b]] for b in live])
             y = torch.zeros((rows.shape[0], W), dtype=TD[dtype], device=DEV)
-            K.mingru_scan(dev(rows), W, state, i32(np.cumsum([0] + [hi[b] - lo[b] for b in live])), i32([b + 1 for b in live]), y)
+            longest = max(hi[b] - lo[b] for b in live)
+            # (steps whose longest sequence has more than 32 tokens take the scan in three passes over runs of 32)
+            runs = torch.zeros(2 * len(live) * -(-longest // 32) * W, dtype=torch.float32, device=DEV)
+            K.mingru_scan(dev(rows), W, state, i32(np.cumsum([0] + [hi[b] - lo[b] for b in live])), i32([b + 1 for b in live]), y,
+                          longest, runs)
             y = y.float().cpu().numpy()
             at = 0
             for b in live:
@@ -367,6 +371,13 @@ def test_norm_per_head_with_gate_and_the_average_of_two_sides(dtype):
     K.sides_norm_add(xd, dev(a), dev(b), dev(wa), dev(wb), 1e-6, 0.35)
     ref = x + 0.35 * (P.rms_norm(a, wa, 1e-6) + P.rms_norm(b, wb, 1e-6))
     np.testing.assert_allclose(xd.cpu().numpy(), ref, atol=1e-5)
+    # with what a folded norm reads: the completed rows' sums of squares, and the rows times the next norm's weight
+    xd, ssq, xg = dev(x), torch.zeros(64, dtype=torch.float32, device=DEV), torch.zeros((T, d), dtype=torch.bfloat16, device=DEV)
+    nw = rng.standard_normal(d).astype(np.float32)
+    K.sides_norm_add(xd, dev(a), dev(b), dev(wa), dev(wb), 1e-6, 0.35, ssq, dev(nw), xg)
+    np.testing.assert_allclose(xd.cpu().numpy(), ref, atol=1e-5)
+    np.testing.assert_allclose(ssq[:T].cpu().numpy(), (ref * ref).sum(1), rtol=1e-5)
+    np.testing.assert_allclose(xg.float().cpu().numpy(), ref * nw, atol=2e-2 * np.abs(ref * nw).max())
 
 
 # ----------------------------------------------------------------- whole models through the engine
