@@ -60,7 +60,7 @@ def _declare(lib):
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, I, P, I, F, I, P],
         "gl3_pair_rows": [P, P, P, P, P, P, L, L, L, L, P, I, P],
         "gl3_concat_rows": [P, P, P, I, I, I, P],
-        "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P],
+        "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
         "gl3_tanh_rows": [P, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
@@ -480,11 +480,13 @@ def concat_rows(a, b, out):
            "concat_rows")
 
 
-def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, gate_col=0):
+def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, gate_col=0, cache=None):
     """Runs of heads inside ``rows`` [T, ld] turned in place by the tokens' positions. ``runs``: up to three of
     ``(first column, heads, head_dim, rot_dim, cos, sin)`` with tables [positions, rot_dim / 2] float32 (None, None: not
     rotated). ``back``: by minus the angle. ``gate`` (one run): rows [T, *] of the same dtype whose column
-    ``gate_col + h`` holds head h's gate; every element of the head is multiplied by its sigmoid."""
+    ``gate_col + h`` holds head h's gate; every element of the head is multiplied by its sigmoid. ``cache``:
+    ``(k_cache, v_cache, table_rows, block_table, page_size)``; the runs are then queries, keys and values, and keys and
+    values also go to the tokens' places in one layer's paged cache."""
     _dev(rows, "rows", contiguous=False); _dev(positions, "positions", torch.int32)
     T = rows.shape[0]
     if rows.dim() != 2 or rows.stride(1) != 1 or positions.numel() != T or not 1 <= len(runs) <= 3:
@@ -505,9 +507,19 @@ def rotate_heads(rows, positions, runs, adjacent=False, back=False, gate=None, g
         if gate.dim() != 2 or gate.shape[0] != T or gate.stride(1) != 1 or n != 1 or gate_col < 0 or gate_col + runs[0][1] > gate.shape[1]:
             raise KernelError(f"rotate_heads: gate {tuple(gate.shape)} from column {gate_col}")
         gate_ld = gate.stride(0)
+    kc = vc = trows = table = None
+    stride = page = 0
+    if cache is not None:
+        kc, vc, trows, table, page = cache
+        _dev(trows, "table_rows", torch.int32); _dev(table, "block_table", torch.int32)
+        _dev(kc, "k_cache", rows.dtype); _dev(vc, "v_cache", rows.dtype)
+        if n != 3 or runs[1][1] != runs[2][1] or trows.numel() != T or table.dim() != 2:
+            raise KernelError("rotate_heads: a cache write takes queries, keys and values and a table row per token")
+        _check_cache(kc, vc, runs[1][1], page, runs[1][2], "rotate_heads", runs[2][2])
+        stride = table.shape[1]
     _check(library().gl3_rotate_heads(_ptr(rows), _code(rows, "rows"), rows.stride(0), _ptr(positions), T, *ints, *tabs, n,
-                                      int(bool(adjacent)), int(bool(back)), _ptr(gate), gate_ld, int(gate_col), _stream()),
-           "rotate_heads")
+                                      int(bool(adjacent)), int(bool(back)), _ptr(gate), gate_ld, int(gate_col), _ptr(kc),
+                                      _ptr(vc), _ptr(trows), _ptr(table), stride, int(page), _stream()), "rotate_heads")
 
 
 def sides_norm_add(x, a, b, wa, wb, eps, factor, ssq=None, next_weight=None, xg=None):

@@ -78,43 +78,63 @@ struct RotRun {
   const float* sin_tab;
 };
 
+// With a cache (k_cache not null; three runs: queries, keys, values) the second and third run also go to the token's
+// place in its page as they come out of the rotation: keys [page][kv head][position][head_dim], values transposed, both
+// in the tiles of gl3_k_offset / gl3_v_offset; page = block_table[table_rows[t] * table_stride + position / page_size].
 template <typename T>
 __global__ __launch_bounds__(64) void rotate_heads_kernel(T* __restrict__ rows, long ld, const int* __restrict__ positions,
                                                            RotRun a, RotRun b, RotRun c, int adjacent, int back,
-                                                           const T* __restrict__ gate, long gate_ld, int gate_col) {
+                                                           const T* __restrict__ gate, long gate_ld, int gate_col,
+                                                           T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                           const int* __restrict__ table_rows,
+                                                           const int* __restrict__ block_table, int table_stride,
+                                                           int page_size) {
   const int t = blockIdx.x;
-  int head = blockIdx.y;
+  int head = blockIdx.y, which = 0;
   RotRun r = a;
   if (head >= a.heads) {
     head -= a.heads;
     r = b;
+    which = 1;
     if (head >= b.heads) {
       head -= b.heads;
       r = c;
+      which = 2;
     }
   }
   const int pos = positions[t];
   T* p = rows + (long)t * ld + r.col + (long)head * r.head_dim;
   const int half = r.rot_dim / 2;
   const float g = gate ? 1.0f / (1.0f + expf(-to_f32<T>(gate[(long)t * gate_ld + gate_col + head]))) : 1.0f;
+  T* dst = nullptr;          // the head's page of the cache, if it goes there
+  const int in_page = pos % page_size;
+  if (k_cache && which > 0) {
+    const long page = block_table[(long)table_rows[t] * table_stride + pos / page_size];
+    dst = (which == 1 ? k_cache : v_cache) + (page * r.heads + head) * (long)page_size * r.head_dim;
+  }
+  auto put = [&](int i, T v) {
+    p[i] = v;
+    if (dst) dst[which == 1 ? gl3_k_offset(in_page, i, r.head_dim) : gl3_v_offset(i, in_page, page_size)] = v;
+  };
   if (r.cos_tab) {
     for (int j = threadIdx.x; j < half; j += 64) {
       const int i0 = adjacent ? 2 * j : j, i1 = adjacent ? 2 * j + 1 : j + half;
       const float cs = r.cos_tab[(long)pos * half + j];
       const float sn = back ? -r.sin_tab[(long)pos * half + j] : r.sin_tab[(long)pos * half + j];
       const float v0 = to_f32<T>(p[i0]), v1 = to_f32<T>(p[i1]);
-      p[i0] = from_f32<T>((v0 * cs - v1 * sn) * g);
-      p[i1] = from_f32<T>((v1 * cs + v0 * sn) * g);
+      put(i0, from_f32<T>((v0 * cs - v1 * sn) * g));
+      put(i1, from_f32<T>((v1 * cs + v0 * sn) * g));
     }
   }
-  if (gate)
-    for (int i = (r.cos_tab ? r.rot_dim : 0) + threadIdx.x; i < r.head_dim; i += 64) p[i] = from_f32<T>(to_f32<T>(p[i]) * g);
+  if (gate || dst)
+    for (int i = (r.cos_tab ? r.rot_dim : 0) + threadIdx.x; i < r.head_dim; i += 64) put(i, from_f32<T>(to_f32<T>(p[i]) * g));
 }
 
 extern "C" int gl3_rotate_heads(void* rows, int dtype, long ld, const int* positions, int n_tokens, const int* cols,
                                 const int* heads, const int* head_dims, const int* rot_dims, const float* const* cos_tabs,
                                 const float* const* sin_tabs, int n_runs, int adjacent, int back, const void* gate,
-                                long gate_ld, int gate_col, hipStream_t stream) {
+                                long gate_ld, int gate_col, void* k_cache, void* v_cache, const int* table_rows,
+                                const int* block_table, int table_stride, int page_size, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(rows && positions && n_tokens > 0 && n_runs >= 1 && n_runs <= 3, "gl3_rotate_heads: bad arguments");
   GL3_REQUIRE(!gate || n_runs == 1, "gl3_rotate_heads: a gate goes with one run of heads");
@@ -129,13 +149,24 @@ extern "C" int gl3_rotate_heads(void* rows, int dtype, long ld, const int* posit
     total += heads[i];
   }
   GL3_REQUIRE(total <= 65535, "gl3_rotate_heads: %ld heads exceed the grid", total);
+  if (k_cache) {
+    GL3_REQUIRE(v_cache && table_rows && block_table && table_stride > 0 && n_runs == 3 && heads[1] == heads[2],
+                "gl3_rotate_heads: a cache write takes queries, keys and values, as many value heads as key heads");
+    GL3_REQUIRE(page_size > 0 && page_size % 32 == 0 && head_dims[1] % 16 == 0 && head_dims[2] % 16 == 0,
+                "gl3_rotate_heads: the cache lies in tiles: page_size %d must be a multiple of 32, head sizes %d and %d of 16",
+                page_size, head_dims[1], head_dims[2]);
+  } else {
+    page_size = 1;
+  }
   dim3 grid(n_tokens, (unsigned)total), block(64);
   if (dtype == GL3_F32)
     rotate_heads_kernel<float><<<grid, block, 0, stream>>>((float*)rows, ld, positions, r[0], r[1], r[2], adjacent, back,
-                                                           (const float*)gate, gate_ld, gate_col);
+                                                           (const float*)gate, gate_ld, gate_col, (float*)k_cache,
+                                                           (float*)v_cache, table_rows, block_table, table_stride, page_size);
   else if (dtype == GL3_BF16)
     rotate_heads_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)rows, ld, positions, r[0], r[1], r[2], adjacent, back,
-                                                            (const bf16_t*)gate, gate_ld, gate_col);
+                                                            (const bf16_t*)gate, gate_ld, gate_col, (bf16_t*)k_cache,
+                                                            (bf16_t*)v_cache, table_rows, block_table, table_stride, page_size);
   else GL3_REQUIRE(false, "gl3_rotate_heads: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;
@@ -447,31 +478,33 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
   }
   const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
   float ld[TM_LD];
-  // item idx of a round: token idx / (4 D), array (idx / D) % 4, element idx % D
-  auto fetch = [&](int tb) {
-    const int n = t1 - tb < ch ? t1 - tb : ch;
+  // item idx = tid + m * nt of a round: token idx / (4 D), array (idx / D) % 4, element idx % D. A thread's items are
+  // the same in every round, so where they come from and go to is worked out once (the divisions are not cheap).
+  const float* from[TM_LD];      // the item's address in the round that starts at token t0
+  int to[TM_LD], token[TM_LD];   // its place in a stage buffer (-1 - place for a decay, which passes the exponentials)
 #pragma unroll
-    for (int m = 0; m < TM_LD; ++m) {
-      const int idx = tid + m * nt;
-      float x = 0.f;
-      if (idx < n * 4 * D) {
-        const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
-        const float* src = a == 0 ? r : a == 1 ? k : a == 2 ? wl : v;
-        x = src[(long)(tb + tt) * HD + (long)head * D + i];
-      }
-      ld[m] = x;
-    }
+  for (int m = 0; m < TM_LD; ++m) {
+    const int idx = tid + m * nt;
+    const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
+    const float* src = a == 0 ? r : a == 1 ? k : a == 2 ? wl : v;
+    from[m] = src + (long)(t0 + tt) * HD + (long)head * D + i;
+    token[m] = tt < ch ? tt : 0x7fffffff;
+    to[m] = (tt * 4 + a) * Dr + i;
+    if (a == 2) to[m] = -1 - to[m];
+  }
+  auto fetch = [&](int tb) {
+    const int n = t1 - tb;
+#pragma unroll
+    for (int m = 0; m < TM_LD; ++m) ld[m] = token[m] < n ? from[m][(long)(tb - t0) * HD] : 0.f;
   };
   auto put = [&](int buf, int tb) {
-    const int n = t1 - tb < ch ? t1 - tb : ch;
+    const int n = t1 - tb;
 #pragma unroll
-    for (int m = 0; m < TM_LD; ++m) {
-      const int idx = tid + m * nt;
-      if (idx < n * 4 * D) {
-        const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
-        stage[((buf * ch + tt) * 4 + a) * Dr + i] = a == 2 ? expf(-expf(ld[m])) : ld[m];
+    for (int m = 0; m < TM_LD; ++m)
+      if (token[m] < n) {
+        if (to[m] >= 0) stage[buf * ch * 4 * Dr + to[m]] = ld[m];
+        else stage[buf * ch * 4 * Dr - 1 - to[m]] = expf(-expf(ld[m]));
       }
-    }
   };
   if (t0 < t1) {
     fetch(t0);

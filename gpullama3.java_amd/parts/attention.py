@@ -192,15 +192,12 @@ class GQAAttention:
         qkv = ctx.buffer("qkvg", (T, self.w_qkv.shape[0]), self.dtype)
         ops.linear(h, self.w_qkv, qkv, ops.EPI_STORE, ctx)
         pos, vpos = self.position, self.value_position
-        runs = []
-        if pos is not None:
-            runs += [(0, H, hs, pos.rot_dim, pos.cos, pos.sin), (qn, Kh, hs, pos.rot_dim, pos.cos, pos.sin)]
-        if vpos is not None:
-            runs.append((qn + kn, Kh, vd, vpos.rot_dim, vpos.cos, vpos.sin))
-        if runs:
-            K.rotate_heads(qkv, ctx.positions, runs, adjacent=bool((pos or vpos).adjacent))
-        K.kv_write(qkv, qn, qn + kn, ctx.positions, ops._table_rows(ctx), table, k_cache, v_cache, Kh, hs, vd,
-                   k_cache.shape[2])
+        # q, k and v turned in place, k and v into the cache as they come out: one kernel
+        qk = (pos.rot_dim, pos.cos, pos.sin) if pos is not None else (0, None, None)
+        vr = (vpos.rot_dim, vpos.cos, vpos.sin) if vpos is not None else (0, None, None)
+        K.rotate_heads(qkv, ctx.positions, [(0, H, hs) + qk, (qn, Kh, hs) + qk, (qn + kn, Kh, vd) + vr],
+                       adjacent=bool(pos.adjacent if pos is not None else vpos is not None and vpos.adjacent),
+                       cache=(k_cache, v_cache, ops._table_rows(ctx), table, k_cache.shape[2]))
         att = ctx.buffer("attn_out", (T, H * vd), self.dtype)
         ops.attention(ctx, qkv, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale, v_head_dim=vd,
                       slopes=self.slopes, sink=self.sink, keep_first=self.keep_first)
