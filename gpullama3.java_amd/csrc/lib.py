@@ -62,10 +62,10 @@ def _declare(lib):
         "gl3_concat_rows": [P, P, P, I, I, I, P],
         "gl3_rotate_heads": [P, I, L, P, I, P, P, P, P, P, P, I, I, I, P, L, I, P, P, P, P, I, I, P],
         "gl3_sides_norm_add": [P, P, P, P, P, F, F, I, I, P, P, P, P],
-        "gl3_tanh_rows": [P, P, I, L, P],
+        "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
         "gl3_shift_mix": [P, I, I, P, I, P, L, P, P, P, P, I, I, I, P],
-        "gl3_timemix": [P, P, P, P, P, P, L, L, P, P, P, I, I, I, P],
+        "gl3_timemix": [P, P, P, L, P, L, P, P, L, L, P, P, P, I, I, I, P, L, P, F, P, I, P],
         "gl3_head_norm_gate": [P, P, P, F, P, I, I, I, I, P],
         "gl3_kv_write": [P, I, L, I, I, P, P, P, I, P, P, I, I, I, I, I, P],
         "gl3_residual_inject": [P, P, P, I, I, P],
@@ -546,11 +546,12 @@ def sides_norm_add(x, a, b, wa, wb, eps, factor, ssq=None, next_weight=None, xg=
 
 
 def tanh_rows(src, out):
-    """out = tanh(src) in ``out``'s dtype (src float32, same number of elements, both contiguous)."""
-    _dev(src, "src", torch.float32); _dev(out, "out")
-    if src.numel() != out.numel():
-        raise KernelError(f"tanh_rows: {src.numel()} inputs for {out.numel()} outputs")
-    _check(library().gl3_tanh_rows(_ptr(src), _ptr(out), _code(out, "out"), src.numel(), _stream()), "tanh_rows")
+    """out = tanh(src) in ``out``'s dtype: src float32 [T, n] (rows may be strided), out [T, n] contiguous."""
+    _dev(src, "src", torch.float32, contiguous=False); _dev(out, "out")
+    if src.dim() != 2 or src.stride(1) != 1 or out.shape != src.shape:
+        raise KernelError(f"tanh_rows: src {tuple(src.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_tanh_rows(_ptr(src), src.stride(0), src.shape[1], _ptr(out), _code(out, "out"), src.numel(),
+                                   _stream()), "tanh_rows")
 
 
 MINGRU_RUN = 32      # tokens of a run of the three-pass scan (MG_RUN in mixers.hip)
@@ -595,20 +596,39 @@ def shift_mix(h, mu, state, cu_seqlens, seq_of_token, slot_ids, out, one_token_e
                                    int(bool(one_token_each)), _stream()), "shift_mix")
 
 
-def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, H, D):
-    """The decayed matrix per head, token by token from the state in each sequence's slot (``mixers.hip``): r, k, v,
-    w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D]; ``out``
-    [T, H D] float32 receives the raw read-outs; ``state`` [slots, >= state_off + H D D] float32."""
-    for t, n in ((r, "r"), (k, "k"), (v, "v"), (w_log, "w_log"), (bonus, "bonus"), (out, "out")):
-        _dev(t, n, torch.float32)
+def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, H, D, gate=None, norm_w=None, eps=0.0,
+            normed=None):
+    """The decayed matrix per head, token by token from the state in each sequence's slot (``mixers.hip``): r, k, v
+    [T, H D] float32 (rows of one common stride), w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D];
+    ``state`` [slots, >= state_off + H D D] float32. ``out`` [T, H D] float32 (may be None) receives the raw read-outs;
+    ``normed`` [T, H D] (may be None; then ``gate`` [T, H D] float32, ``norm_w`` [H D] float32 and ``eps``) receives
+    read-out / rms per head * norm_w * silu(gate)."""
+    for t, n in ((r, "r"), (k, "k"), (v, "v"), (w_log, "w_log")):
+        _dev(t, n, torch.float32, contiguous=False)
+    _dev(bonus, "bonus", torch.float32)
     _dev(state, "state", torch.float32, contiguous=False)
     _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(slot_ids, "slot_ids", torch.int32)
     T, B = r.shape[0], slot_ids.numel()
-    if (any(t.shape != (T, H * D) for t in (r, k, v, w_log, out)) or bonus.numel() != H * D or state.dim() != 2
+    if (any(t.shape != (T, H * D) or t.stride(1) != 1 for t in (r, k, v, w_log)) or not r.stride(0) == k.stride(0) == v.stride(0)
+            or bonus.numel() != H * D or state.dim() != 2
             or state.shape[1] < state_off + H * D * D or state.stride(1) != 1 or cu_seqlens.numel() != B + 1):
         raise KernelError(f"timemix: r {tuple(r.shape)} for {H} heads of {D}, state {tuple(state.shape)}")
-    _check(library().gl3_timemix(_ptr(r), _ptr(k), _ptr(v), _ptr(w_log), _ptr(bonus), _ptr(state), state.stride(0),
-                                 int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out), B, H, D, _stream()), "timemix")
+    if out is None and normed is None:
+        raise KernelError("timemix: nothing to write to")
+    if out is not None:
+        _dev(out, "out", torch.float32)
+        if out.shape != (T, H * D):
+            raise KernelError(f"timemix: out {tuple(out.shape)}")
+    ld_g = 0
+    if normed is not None:
+        _dev(normed, "normed"); _dev(gate, "gate", torch.float32, contiguous=False); _dev(norm_w, "norm_w", torch.float32)
+        if normed.shape != (T, H * D) or gate.shape != (T, H * D) or gate.stride(1) != 1 or norm_w.numel() != H * D:
+            raise KernelError(f"timemix: normed {tuple(normed.shape)}, gate {tuple(gate.shape)}, weight {tuple(norm_w.shape)}")
+        ld_g = gate.stride(0)
+    _check(library().gl3_timemix(_ptr(r), _ptr(k), _ptr(v), r.stride(0), _ptr(w_log), w_log.stride(0), _ptr(bonus),
+                                 _ptr(state), state.stride(0), int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
+                                 B, H, D, _ptr(gate), ld_g, _ptr(norm_w), float(eps), _ptr(normed),
+                                 _code(normed, "normed") if normed is not None else F32, _stream()), "timemix")
 
 
 def head_norm_gate(o, weight, gate, eps, out, H, D):

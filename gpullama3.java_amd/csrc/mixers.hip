@@ -227,18 +227,19 @@ extern "C" int gl3_sides_norm_add(float* x, const float* a, const float* b, cons
 }
 
 // ----------------------------------------------------------------- out = tanh(in) in the activations' type
+// in: rows of `ld` floats, `cols` of them used; out: [rows][cols] contiguous
 template <typename T>
-__global__ void tanh_rows_kernel(const float* __restrict__ in, T* __restrict__ out, long n) {
+__global__ void tanh_rows_kernel(const float* __restrict__ in, long ld, int cols, T* __restrict__ out, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) out[i] = from_f32<T>(tanhf(in[i]));
+  if (i < n) out[i] = from_f32<T>(tanhf(in[(i / cols) * ld + i % cols]));
 }
 
-extern "C" int gl3_tanh_rows(const float* in, void* out, int out_dtype, long n, hipStream_t stream) {
+extern "C" int gl3_tanh_rows(const float* in, long ld, int cols, void* out, int out_dtype, long n, hipStream_t stream) {
   if (n == 0) return 0;
-  GL3_REQUIRE(in && out && n > 0 && (n + 255) / 256 < (1L << 31), "gl3_tanh_rows: bad arguments");
+  GL3_REQUIRE(in && out && n > 0 && cols > 0 && ld >= cols && (n + 255) / 256 < (1L << 31), "gl3_tanh_rows: bad arguments");
   const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-  if (out_dtype == GL3_F32) tanh_rows_kernel<float><<<grid, block, 0, stream>>>(in, (float*)out, n);
-  else if (out_dtype == GL3_BF16) tanh_rows_kernel<bf16_t><<<grid, block, 0, stream>>>(in, (bf16_t*)out, n);
+  if (out_dtype == GL3_F32) tanh_rows_kernel<float><<<grid, block, 0, stream>>>(in, ld, cols, (float*)out, n);
+  else if (out_dtype == GL3_BF16) tanh_rows_kernel<bf16_t><<<grid, block, 0, stream>>>(in, ld, cols, (bf16_t*)out, n);
   else GL3_REQUIRE(false, "gl3_tanh_rows: unknown dtype %d", out_dtype);
   GL3_LAUNCH_CHECK();
   return 0;
@@ -449,14 +450,19 @@ extern "C" int gl3_shift_mix(const void* h, int dtype, int d, const float* mu, i
 #define TM_MAXD 256
 #define TM_LD 8           // loads a thread has on their way for the next round
 
-template <int RP>
+// r, k, v are rows of `ld` floats, wl rows of `ld_w` (a token's H*D values from the pointer on). o (may be null): the raw
+// read-outs [T][H*D]. out (may be null; then gate, rows of `ld_g`, and norm_w [H*D]): at the end of a round one wave a
+// token divides the head's read-out by its root mean square and multiplies by the weight per channel and silu(gate):
+// out[t, h, i] = o / sqrt(mean_i(o^2) + eps) * norm_w[h*D + i] * silu(gate[t, h*D + i]), in the activations' type.
+template <int RP, typename TO>
 __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__ r, const float* __restrict__ k,
-                                                        const float* __restrict__ v, const float* __restrict__ wl,
-                                                        const float* __restrict__ bonus, float* __restrict__ state,
+                                                        const float* __restrict__ v, long ld, const float* __restrict__ wl,
+                                                        long ld_w, const float* __restrict__ bonus, float* __restrict__ state,
                                                         long state_stride, long state_off,
                                                         const int* __restrict__ cu_seqlens,
                                                         const int* __restrict__ slot_ids, float* __restrict__ o, int H,
-                                                        int D, int ch) {
+                                                        int D, int ch, const float* __restrict__ gate, long ld_g,
+                                                        const float* __restrict__ norm_w, float eps, TO* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) float tm_shared[];
   const int head = blockIdx.x, seq = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -477,17 +483,19 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
     ub[ii] = i0 + ii < D ? bonus[head * D + i0 + ii] : 0.f;
   }
   const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
-  float ld[TM_LD];
+  float ld_[TM_LD];
   // item idx = tid + m * nt of a round: token idx / (4 D), array (idx / D) % 4, element idx % D. A thread's items are
   // the same in every round, so where they come from and go to is worked out once (the divisions are not cheap).
   const float* from[TM_LD];      // the item's address in the round that starts at token t0
   int to[TM_LD], token[TM_LD];   // its place in a stage buffer (-1 - place for a decay, which passes the exponentials)
+  long step[TM_LD];              // floats from a token's row to the next token's
 #pragma unroll
   for (int m = 0; m < TM_LD; ++m) {
     const int idx = tid + m * nt;
     const int tt = idx / (4 * D), rest = idx - tt * 4 * D, a = rest / D, i = rest - a * D;
     const float* src = a == 0 ? r : a == 1 ? k : a == 2 ? wl : v;
-    from[m] = src + (long)(t0 + tt) * HD + (long)head * D + i;
+    from[m] = src + (long)(t0 + tt) * (a == 2 ? ld_w : ld) + (long)head * D + i;
+    step[m] = a == 2 ? ld_w : ld;
     token[m] = tt < ch ? tt : 0x7fffffff;
     to[m] = (tt * 4 + a) * Dr + i;
     if (a == 2) to[m] = -1 - to[m];
@@ -495,15 +503,15 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
   auto fetch = [&](int tb) {
     const int n = t1 - tb;
 #pragma unroll
-    for (int m = 0; m < TM_LD; ++m) ld[m] = token[m] < n ? from[m][(long)(tb - t0) * HD] : 0.f;
+    for (int m = 0; m < TM_LD; ++m) ld_[m] = token[m] < n ? from[m][(long)(tb - t0) * step[m]] : 0.f;
   };
   auto put = [&](int buf, int tb) {
     const int n = t1 - tb;
 #pragma unroll
     for (int m = 0; m < TM_LD; ++m)
       if (token[m] < n) {
-        if (to[m] >= 0) stage[buf * ch * 4 * Dr + to[m]] = ld[m];
-        else stage[buf * ch * 4 * Dr - 1 - to[m]] = expf(-expf(ld[m]));
+        if (to[m] >= 0) stage[buf * ch * 4 * Dr + to[m]] = ld_[m];
+        else stage[buf * ch * 4 * Dr - 1 - to[m]] = expf(-expf(ld_[m]));
       }
   };
   if (t0 < t1) {
@@ -543,7 +551,23 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
       const int tt = idx / D, jj = idx - tt * D;
       float sum = 0.f;
       for (int p = 0; p < P; ++p) sum += parts[(buf * ch + tt) * P * cols + p * cols + jj];
-      o[(long)(tb + tt) * HD + (long)head * D + jj] = sum;
+      if (o) o[(long)(tb + tt) * HD + (long)head * D + jj] = sum;
+      if (out) parts[(buf * ch + tt) * P * cols + jj] = sum;      // (the first part's place: only this thread reads it)
+    }
+    if (out) {
+      __syncthreads();
+      for (int tt = wave; tt < n; tt += nt >> 6) {
+        const float* sums = parts + (buf * ch + tt) * P * cols;
+        float ss = 0.f;
+        for (int i = lane; i < D; i += 64) ss += sums[i] * sums[i];
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+        for (int i = lane; i < D; i += 64) {
+          const float g = gate[(long)(tb + tt) * ld_g + (long)head * D + i];
+          out[(long)(tb + tt) * HD + (long)head * D + i] =
+              from_f32<TO>(sums[i] * inv * norm_w[head * D + i] * (g / (1.0f + expf(-g))));
+        }
+      }
     }
   }
 #pragma unroll
@@ -554,13 +578,17 @@ __global__ __launch_bounds__(1024) void timemix_kernel(const float* __restrict__
 // rows a wave owns: 8 for heads of up to 64 (eight waves a head), 16 up to 128, 64 beyond
 static int timemix_rows(int D) { return D <= 64 ? 8 : D <= 128 ? 16 : 64; }
 
-extern "C" int gl3_timemix(const float* r, const float* k, const float* v, const float* wl, const float* bonus,
-                           float* state, long state_stride, long state_off, const int* cu_seqlens, const int* slot_ids,
-                           float* o, int n_seqs, int H, int D, hipStream_t stream) {
+extern "C" int gl3_timemix(const float* r, const float* k, const float* v, long ld, const float* wl, long ld_w,
+                           const float* bonus, float* state, long state_stride, long state_off, const int* cu_seqlens,
+                           const int* slot_ids, float* o, int n_seqs, int H, int D, const float* gate, long ld_g,
+                           const float* norm_w, float eps, void* out, int out_dtype, hipStream_t stream) {
   if (n_seqs == 0) return 0;
-  GL3_REQUIRE(r && k && v && wl && bonus && state && cu_seqlens && slot_ids && o && n_seqs > 0 && n_seqs <= 65535 && H > 0,
-              "gl3_timemix: bad arguments");
+  GL3_REQUIRE(r && k && v && wl && bonus && state && cu_seqlens && slot_ids && (o || out) && n_seqs > 0 && n_seqs <= 65535 &&
+                  H > 0, "gl3_timemix: bad arguments");
   GL3_REQUIRE(D >= 1 && D <= TM_MAXD, "gl3_timemix: heads of %d elements: the kernel holds up to %d", D, TM_MAXD);
+  GL3_REQUIRE(ld >= (long)H * D && ld_w >= (long)H * D, "gl3_timemix: rows of %ld and %ld floats for %d heads of %d", ld, ld_w, H, D);
+  GL3_REQUIRE(!out || (gate && norm_w && ld_g >= (long)H * D && (out_dtype == GL3_F32 || out_dtype == GL3_BF16)),
+              "gl3_timemix: the read-outs' norm needs the gate, the weight and an output of a known type");
   GL3_REQUIRE(state_off >= 0 && state_off + (long)H * D * D <= state_stride, "gl3_timemix: the state's row of %ld floats", state_stride);
   dim3 grid(H, n_seqs);
   const int RP = timemix_rows(D), CG = (D + 63) / 64, P = (D + RP - 1) / RP;
@@ -571,12 +599,17 @@ extern "C" int gl3_timemix(const float* r, const float* k, const float* v, const
   if (ch > 16) ch = 16;
   GL3_REQUIRE(ch >= 1 && nt <= 1024, "gl3_timemix: heads of %d do not fit the kernel's shared memory", D);
   const size_t shared = (size_t)ch * per_token * sizeof(float);
-#define TM_GO(R) timemix_kernel<R><<<grid, dim3(nt), shared, stream>>>(r, k, v, wl, bonus, state, state_stride, state_off, \
-                                                                   cu_seqlens, slot_ids, o, H, D, ch)
+#define TM_ARGS r, k, v, ld, wl, ld_w, bonus, state, state_stride, state_off, cu_seqlens, slot_ids, o, H, D, ch, gate, ld_g, norm_w, eps
+#define TM_GO(R)                                                                                                    \
+  do {                                                                                                              \
+    if (out && out_dtype == GL3_BF16) timemix_kernel<R, bf16_t><<<grid, dim3(nt), shared, stream>>>(TM_ARGS, (bf16_t*)out); \
+    else timemix_kernel<R, float><<<grid, dim3(nt), shared, stream>>>(TM_ARGS, (float*)out);                       \
+  } while (0)
   if (RP == 8) TM_GO(8);
   else if (RP == 16) TM_GO(16);
   else TM_GO(64);
 #undef TM_GO
+#undef TM_ARGS
   GL3_LAUNCH_CHECK();
   return 0;
 }

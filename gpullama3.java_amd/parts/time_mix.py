@@ -9,7 +9,10 @@ head, with S [head_dim, head_dim] in 32-bit::
 
 (the bonus u counts for the current token only). Each head's o is divided by its root mean square, multiplied by a
 weight per channel and by the gate, and goes through the output projection. The projections' sums stay in 32-bit,
-and so does everything behind them. A sequence's state (its last h, then the heads' matrices) lives in the cache's
+and so does everything behind them. The rows of W_r, W_k, W_v, W_g and W_w1 are stacked: a step of few tokens makes
+all five projections with ONE product over the five blends stacked by rows (every blend meets every matrix; the
+kernels read the five blocks on the diagonal; the weights, which are what such a step waits for, are read once), a
+prompt makes five products over the stored matrices. A sequence's state (its last h, then the heads' matrices) lives in the cache's
 per-slot state, zeroed when the slot is handed out; the kernels (``csrc/mixers.hip``) walk a step's tokens in order
 from it, so every cut of a sequence into steps gives the same result.
 """
@@ -52,7 +55,17 @@ class TimeMix:
     def load(self, weights):
         n = self.names
         without = getattr(self, "without", frozenset())
-        self.w = {s: ops.for_few_rows(weights[n[s]], without=without) for s in ("r", "k", "v", "g", "w1", "w2")}
+        parts = [weights[n[s]] for s in ("r", "k", "v", "g", "w1")]
+        dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
+        rows = sum(p.shape[0] for p in parts)
+        pad = torch.zeros((-(-rows // 16) * 16 - rows, self.d), dtype=dt, device=parts[0].device)
+        self.w_all = ops.for_few_rows(torch.cat([p.to(dt) for p in parts] + [pad], dim=0).contiguous(), without=without)
+        lo = 0
+        self.w = {}
+        for s, p in zip(("r", "k", "v", "g", "w1"), parts):      # the stored names stay addressable as views
+            self.w[s] = weights[n[s]] = self.w_all[lo:lo + p.shape[0]]
+            lo += p.shape[0]
+        self.w["w2"] = ops.for_few_rows(weights[n["w2"]], without=without)
         self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
         # what the kernels behind the projections read is kept in 32-bit
         self.mu = torch.stack([weights[n["mu_" + s]].float() for s in _BLENDS]).contiguous()
@@ -76,18 +89,35 @@ class TimeMix:
         blends = ctx.buffer("timemix_blends", (len(_BLENDS), T, d), self.dtype)
         K.shift_mix(h, self.mu, state, ctx.cu_seqlens, ctx.seq_of_token, ctx.slot_ids, blends,
                     one_token_each=bool(ctx.decode and ctx.max_q_len == 1))
-        proj = ctx.buffer("timemix_proj", (5, T, H * D), torch.float32)        # r, k, v, gate, log-decay
-        for i, s in enumerate(("r", "k", "v", "g")):
-            ops.linear(blends[i], self.w[s], proj[i], ops.EPI_STORE, ctx)
-        inner = ctx.buffer("timemix_decay_inner", (T, self.rank), torch.float32)
-        ops.linear(blends[4], self.w["w1"], inner, ops.EPI_STORE, ctx)
+        HD = H * D
+        if 5 * T <= ops.CHUNK_ROWS and self.dtype == torch.bfloat16:
+            # few tokens: one product of all five blends with all five matrices; block (s, s) is projection s
+            both = ctx.buffer("timemix_all", (5 * T, self.w_all.shape[0]), torch.float32)
+            ops.linear(blends.view(5 * T, d), self.w_all, both, ops.EPI_STORE, ctx)
+            r, k, v, g = (both[i * T:(i + 1) * T, i * HD:(i + 1) * HD] for i in range(4))
+            inner = both[4 * T:5 * T, 4 * HD:4 * HD + self.rank]
+        else:
+            proj = ctx.buffer("timemix_proj", (4, T, HD), torch.float32)        # r, k, v, gate
+            for i, s in enumerate(("r", "k", "v", "g")):
+                ops.linear(blends[i], self.w[s], proj[i], ops.EPI_STORE, ctx)
+            r, k, v, g = proj[0], proj[1], proj[2], proj[3]
+            inner = ctx.buffer("timemix_decay_inner", (T, self.rank), torch.float32)
+            ops.linear(blends[4], self.w["w1"], inner, ops.EPI_STORE, ctx)
         squashed = ctx.buffer("timemix_decay_tanh", (T, self.rank), self.dtype)
         K.tanh_rows(inner, squashed)
-        ops.linear(squashed, self.w["w2"], proj[4], ops.EPI_STORE, ctx, bias=self.w0)
-        o = ctx.buffer("timemix_readout", (T, H * D), torch.float32)
-        K.timemix(proj[0], proj[1], proj[2], proj[4], self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, o, H, D)
-        y = ctx.buffer("timemix_out", (T, H * D), self.dtype)
-        K.head_norm_gate(o, self.norm_w, proj[3], self.spec.norm_eps, y, H, D)
+        w_log = ctx.buffer("timemix_decay_log", (T, HD), torch.float32)
+        ops.linear(squashed, self.w["w2"], w_log, ops.EPI_STORE, ctx, bias=self.w0)
+        y = ctx.buffer("timemix_out", (T, HD), self.dtype)
+        if ctx.max_q_len <= 16 or not g.is_contiguous():
+            # the recurrence, and at the end of its round the read-outs' norm per head with weight and gate: one launch
+            K.timemix(r, k, v, w_log, self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, None, H, D,
+                      gate=g, norm_w=self.norm_w, eps=self.spec.norm_eps, normed=y)
+        else:
+            # a prompt: a second barrier in every round of the chain costs more than a kernel that does all norms at once
+            # (2,048 tokens, 32 heads of 64: 8 layers 10.8 against 12.5 ms)
+            o = ctx.buffer("timemix_readout", (T, HD), torch.float32)
+            K.timemix(r, k, v, w_log, self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, o, H, D)
+            K.head_norm_gate(o, self.norm_w, g, self.spec.norm_eps, y, H, D)
         ops.linear(y, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)
 
 

@@ -292,6 +292,8 @@ def test_decayed_matrix_whole_and_in_pieces(H, D):
     r, k, v = (rng.standard_normal((T, H * D)).astype(np.float32) * 0.5 for _ in range(3))
     wl = rng.uniform(-5.0, 0.5, (T, H * D)).astype(np.float32)
     bonus = rng.standard_normal((H, D)).astype(np.float32)
+    gate = rng.standard_normal((T, H * D)).astype(np.float32)
+    norm_w = rng.standard_normal(H * D).astype(np.float32)
     cu = np.cumsum([0] + lens)
     refs = [P.decayed_outer_scan(*(a[lo:hi].reshape(-1, H, D) for a in (r, k, v)),
                                  np.exp(-np.exp(wl[lo:hi].astype(np.float64))).reshape(-1, H, D), bonus,
@@ -308,9 +310,19 @@ def test_decayed_matrix_whole_and_in_pieces(H, D):
             pick = lambda a: dev(np.concatenate([a[cu[b] + lo[b]:cu[b] + hi[b]] for b in live]))
             n_rows = sum(hi[b] - lo[b] for b in live)
             o = torch.zeros((n_rows, H * D), dtype=torch.float32, device=DEV)
-            K.timemix(pick(r), pick(k), pick(v), pick(wl), dev(bonus), state, off,
-                      i32(np.cumsum([0] + [hi[b] - lo[b] for b in live])), i32([b for b in live]), o, H, D)
+            # (r, k, v as columns of wider rows, as the stacked product of a short step leaves them; with the read-outs'
+            # norm, weight and gate at the end of every round)
+            wide = torch.zeros((n_rows, 3 * H * D + 8), dtype=torch.float32, device=DEV)
+            for i, a in enumerate((r, k, v)):
+                wide[:, i * H * D:(i + 1) * H * D] = pick(a)
+            normed = torch.zeros((n_rows, H * D), dtype=torch.float32, device=DEV)
+            K.timemix(wide[:, :H * D], wide[:, H * D:2 * H * D], wide[:, 2 * H * D:3 * H * D], pick(wl), dev(bonus), state, off,
+                      i32(np.cumsum([0] + [hi[b] - lo[b] for b in live])), i32([b for b in live]), o, H, D,
+                      gate=pick(gate), norm_w=dev(norm_w), eps=1e-4, normed=normed)
             o = o.cpu().numpy()
+            ref_n = (P.rms_unit(o.reshape(-1, H, D), 1e-4).reshape(-1, H * D) * norm_w
+                     * P.silu(np.concatenate([gate[cu[b] + lo[b]:cu[b] + hi[b]] for b in live]).astype(np.float64)))
+            np.testing.assert_allclose(normed.cpu().numpy(), ref_n, atol=1e-4 * max(1.0, np.abs(ref_n).max()))
             at = 0
             for b in live:
                 out[b][lo[b]:hi[b]] = o[at:at + hi[b] - lo[b]]
