@@ -47,9 +47,9 @@ LOOPED = {
     "loop": {"start": 0, "stop": 2, "times": 3},
 }
 # no loop and no soft cap; a minGRU first; an attention that sees every earlier key; one kv head for six heads;
-# a residual factor of one; multipliers so large that their products need 64 bits
+# a residual factor of one; multipliers so large that their products need 64 bits; a width that no tile divides
 STRAIGHT = {
-    "architecture": "Nodupel", "vocab": 203, "width": 72, "norm": {"eps": 1e-6}, "residual_mult": 1.0,
+    "architecture": "Nodupel", "vocab": 203, "width": 100, "norm": {"eps": 1e-6}, "residual_mult": 1.0,
     "embedding": _emb(1.0, 97, 2000000011, 1999999973),
     "layers": [_mingru(40, 100), _parallel(_left(6, 1, 16, 32, 0.3, 20000.0, 8, 1.5), 1, 64, 64),
                _mingru(100, None), _parallel(_left(3, 3, 48, 16, 0.12, 10000.0, 48, None, 70, 3), 4, 16, 96)],
@@ -59,8 +59,8 @@ STRAIGHT = {
 LOOP_AT_END = {
     "architecture": "Nodupel", "vocab": 128, "width": 64, "norm": {"eps": 1e-5}, "residual_mult": 0.45,
     "logit_softcap": 8.0, "embedding": _emb(4.0, 64, 5, 3),
-    "layers": [_parallel(_left(2, 1, 32, 32, 0.2, 1000.0, 32, 8.0, 9, 70), 2, 32, 96), _mingru(64, 96),
-               _parallel(_left(4, 2, 16, 16, 0.3, 10000.0, 4, None, 33, 12), 1, 48, None)],
+    "layers": [_parallel(_left(2, 1, 32, 32, 0.2, 1000.0, 32, 8.0, 9, 70), 2, 32, 96), _mingru(50, 96),
+               _parallel(_left(4, 2, 16, 16, 0.3, 10000.0, 4, None, 33, 12), 3, 20, None)],
     "loop": {"start": 1, "stop": 3, "times": 1},
 }
 # head sizes that the matrix-core attention kernels are built for, widths in whole tiles: what a bfloat16 engine

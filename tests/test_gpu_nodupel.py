@@ -526,3 +526,34 @@ def test_the_command_line_takes_the_model(capsys):
         assert t == int(np.argmax(P.forward(cfg, W, seq)[-1]))
         seq.append(t)
     assert len(got) >= 3
+
+
+def test_the_trace_runner_replays_a_model_of_this_design(tmp_path):
+    """bin/trace_run as a user drives it: a request whole, one with its last tokens one by one, two of unequal lengths
+    in one batch that end at different times; the model class comes from the folder's config.json."""
+    from test_gpu_replay import Replay
+    name = "loop_at_end"
+    folder, cfg, W = model(name)
+    V = cfg["vocab"]
+    reqs = {"a": tokens(name, 50, 90), "b": tokens(name, 51, 140), "c": tokens(name, 52, 7)}
+    ref = {k: P.forward(cfg, W, t) for k, t in reqs.items()}
+    rp = Replay(folder, "float32", tmp_path, max_tokens=400)
+    t = reqs["a"]
+    close(rp.step([("a", t, list(range(len(t))))], end=["a"]).reshape(-1, V), ref["a"], "float32", "whole")
+    t = reqs["b"]
+    rows = [rp.step([("b", t[:100], [0, 50, 99])]).reshape(-1, V)]
+    for j in range(100, len(t)):
+        rows.append(rp.step([("b", [t[j]], [0])], end=["b"] if j == len(t) - 1 else []).reshape(-1, V))
+    close(np.concatenate(rows), ref["b"][[0, 50, 99] + list(range(100, len(t)))], "float32", "decoded")
+    got = {"a": [], "c": []}
+    out = rp.step([("c", reqs["c"][:3], [0, 1, 2]), ("a", reqs["a"][:70], [69])]).reshape(-1, V)
+    got["c"].append(out[:3]); got["a"].append(out[3:])
+    for j in range(20):
+        live = [k for k in ("c", "a") if (3 if k == "c" else 70) + j < len(reqs[k])]
+        at = {k: (3 if k == "c" else 70) + j for k in live}
+        out = rp.step([(k, [reqs[k][at[k]]], [0]) for k in live], end=[k for k in live if at[k] + 1 == len(reqs[k])]).reshape(-1, V)
+        for r, k in enumerate(live):
+            got[k].append(out[r:r + 1])
+    close(np.concatenate(got["c"]), ref["c"], "float32", "the shorter of a batch")
+    close(np.concatenate(got["a"]), ref["a"][69:90], "float32", "the longer of a batch")
+    rp.close()

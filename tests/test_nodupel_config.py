@@ -69,7 +69,7 @@ def test_cache_and_state_needs():
     assert len(kv) == len(state) == len(c.run_order()) + 1          # the last one holds every sequence's previous token
     assert state[-1].elements == 1 and state[-1].dtype == torch.int32
     assert kv[0].keep_first == 70 and kv[0].window == 9 and kv[1] is None
-    assert state[1].elements == 64                                     # the minGRU's channels
+    assert state[1].elements == 50                                     # the minGRU's channels
     assert state[0].elements >= 64 + 2 * 32 * 32                       # the held row and two heads' matrices
 
 
