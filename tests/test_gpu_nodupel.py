@@ -283,7 +283,7 @@ def test_blends_read_the_previous_token_across_steps(dtype):
 
 
 # ----------------------------------------------------------------- the decayed matrix per head
-@pytest.mark.parametrize("H, D", [(3, 24), (2, 48), (1, 64), (2, 100), (1, 128), (1, 200)])
+@pytest.mark.parametrize("H, D", [(3, 24), (2, 48), (1, 64), (2, 100), (1, 128), (1, 200), (2, 8), (1, 256)])
 def test_decayed_matrix_whole_and_in_pieces(H, D):
     from gpullama3_java_amd.csrc import lib as K
     rng = np.random.default_rng([H, D])
