@@ -65,7 +65,7 @@ def _declare(lib):
         "gl3_tanh_rows": [P, L, I, P, I, L, P],
         "gl3_mingru_scan": [P, L, I, P, L, P, P, P, I, I, I, P, P],
         "gl3_shift_mix": [P, I, I, P, I, P, L, P, P, P, P, I, I, I, P],
-        "gl3_timemix": [P, P, P, L, P, L, P, P, L, L, P, P, P, I, I, I, P, L, P, F, P, I, P],
+        "gl3_timemix": [P, P, P, L, P, L, P, P, L, L, P, P, P, I, I, I, P, L, P, F, P, I, I, P],
         "gl3_head_norm_gate": [P, P, P, F, P, I, I, I, I, P],
         "gl3_kv_write": [P, I, L, I, I, P, P, P, I, P, P, I, I, I, I, I, P],
         "gl3_residual_inject": [P, P, P, I, I, P],
@@ -597,12 +597,13 @@ def shift_mix(h, mu, state, cu_seqlens, seq_of_token, slot_ids, out, one_token_e
 
 
 def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, H, D, gate=None, norm_w=None, eps=0.0,
-            normed=None):
+            normed=None, max_q_len=0):
     """The decayed matrix per head, token by token from the state in each sequence's slot (``mixers.hip``): r, k, v
     [T, H D] float32 (rows of one common stride), w_log [T, H D] float32 (the decay is exp(-exp(w_log))), bonus [H, D];
     ``state`` [slots, >= state_off + H D D] float32. ``out`` [T, H D] float32 (may be None) receives the raw read-outs;
     ``normed`` [T, H D] (may be None; then ``gate`` [T, H D] float32, ``norm_w`` [H D] float32 and ``eps``) receives
-    read-out / rms per head * norm_w * silu(gate)."""
+    read-out / rms per head * norm_w * silu(gate). ``max_q_len`` (0: unknown): the most tokens a sequence brings; the
+    kernel's rounds, and with them a block's shared memory, are no longer than that."""
     for t, n in ((r, "r"), (k, "k"), (v, "v"), (w_log, "w_log")):
         _dev(t, n, torch.float32, contiguous=False)
     _dev(bonus, "bonus", torch.float32)
@@ -628,7 +629,7 @@ def timemix(r, k, v, w_log, bonus, state, state_off, cu_seqlens, slot_ids, out, 
     _check(library().gl3_timemix(_ptr(r), _ptr(k), _ptr(v), r.stride(0), _ptr(w_log), w_log.stride(0), _ptr(bonus),
                                  _ptr(state), state.stride(0), int(state_off), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(out),
                                  B, H, D, _ptr(gate), ld_g, _ptr(norm_w), float(eps), _ptr(normed),
-                                 _code(normed, "normed") if normed is not None else F32, _stream()), "timemix")
+                                 _code(normed, "normed") if normed is not None else F32, int(max_q_len), _stream()), "timemix")
 
 
 def head_norm_gate(o, weight, gate, eps, out, H, D):

@@ -581,7 +581,7 @@ static int timemix_rows(int D) { return D <= 64 ? 8 : D <= 128 ? 16 : 64; }
 extern "C" int gl3_timemix(const float* r, const float* k, const float* v, long ld, const float* wl, long ld_w,
                            const float* bonus, float* state, long state_stride, long state_off, const int* cu_seqlens,
                            const int* slot_ids, float* o, int n_seqs, int H, int D, const float* gate, long ld_g,
-                           const float* norm_w, float eps, void* out, int out_dtype, hipStream_t stream) {
+                           const float* norm_w, float eps, void* out, int out_dtype, int max_q_len, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   GL3_REQUIRE(r && k && v && wl && bonus && state && cu_seqlens && slot_ids && (o || out) && n_seqs > 0 && n_seqs <= 65535 &&
                   H > 0, "gl3_timemix: bad arguments");
@@ -597,6 +597,9 @@ extern "C" int gl3_timemix(const float* r, const float* k, const float* v, long 
   int ch = 15360 / per_token;
   if (ch > TM_LD * nt / (4 * D)) ch = TM_LD * nt / (4 * D);
   if (ch > 16) ch = 16;
+  // (max_q_len > 0: no sequence brings more tokens than that; a decode step's blocks then ask for a round of one token's
+  // shared memory, and a CU holds as many of them as its registers allow, not two)
+  if (max_q_len > 0 && ch > max_q_len) ch = max_q_len;
   GL3_REQUIRE(ch >= 1 && nt <= 1024, "gl3_timemix: heads of %d do not fit the kernel's shared memory", D);
   const size_t shared = (size_t)ch * per_token * sizeof(float);
 #define TM_ARGS r, k, v, ld, wl, ld_w, bonus, state, state_stride, state_off, cu_seqlens, slot_ids, o, H, D, ch, gate, ld_g, norm_w, eps

@@ -111,12 +111,13 @@ class TimeMix:
         if ctx.max_q_len <= 16 or not g.is_contiguous():
             # the recurrence, and at the end of its round the read-outs' norm per head with weight and gate: one launch
             K.timemix(r, k, v, w_log, self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, None, H, D,
-                      gate=g, norm_w=self.norm_w, eps=self.spec.norm_eps, normed=y)
+                      gate=g, norm_w=self.norm_w, eps=self.spec.norm_eps, normed=y, max_q_len=ctx.max_q_len)
         else:
             # a prompt: a second barrier in every round of the chain costs more than a kernel that does all norms at once
             # (2,048 tokens, 32 heads of 64: 8 layers 10.8 against 12.5 ms)
             o = ctx.buffer("timemix_readout", (T, HD), torch.float32)
-            K.timemix(r, k, v, w_log, self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, o, H, D)
+            K.timemix(r, k, v, w_log, self.bonus, state, self.state_off, ctx.cu_seqlens, ctx.slot_ids, o, H, D,
+                      max_q_len=ctx.max_q_len)
             K.head_norm_gate(o, self.norm_w, g, self.spec.norm_eps, y, H, D)
         ops.linear(y, self.w_o, x, epilogue, ctx, col_scale=self.out_scale)
 

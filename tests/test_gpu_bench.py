@@ -77,9 +77,11 @@ def test_bench_batch_64_and_a_prefill_of_8192_with_the_8b_layers():
     assert d["prefill"]["tokens"] == 8192 and d["points"] == {}
 
 
-def test_bench_melizen_beside_llama_layers_of_equal_size():
-    """``--arch melizen``: one line of the same outer form, with both models' prefill and decode and their ratio."""
-    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--arch", "melizen", "--layers", "2", "--steps", "3",
+@pytest.mark.parametrize("arch", ["melizen", "nodupel"])
+def test_bench_another_design_beside_llama_layers_of_equal_size(arch):
+    """``--arch melizen`` / ``--arch nodupel``: one line of the same outer form, with both models' prefill and decode
+    and their ratio."""
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--arch", arch, "--layers", "2", "--steps", "3",
                           "--warmup", "2", "--prefill-len", "300", "--prompt-len", "70"], capture_output=True, text=True,
                          timeout=600)
     assert out.returncode == 0, out.stderr[-2000:]
@@ -87,15 +89,15 @@ def test_bench_melizen_beside_llama_layers_of_equal_size():
     assert len(lines) == 1
     d = json.loads(lines[0])
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
-                "vs_baseline", "dtype", "data", "config", "melizen", "llama_of_equal_size", "melizen_over_llama"):
+                "vs_baseline", "dtype", "data", "config", arch, "llama_of_equal_size", f"{arch}_over_llama"):
         assert key in d, key
-    assert d["n_gpus"] == 1 and d["steps"] == 3 and d["warmup"] == 2 and d["dtype"] == "bf16" and "Melizen" in d["metric"]
+    assert d["n_gpus"] == 1 and d["steps"] == 3 and d["warmup"] == 2 and d["dtype"] == "bf16" and arch.capitalize() in d["metric"]
     cfg = d["config"]
     assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
     assert cfg["layers"] == 2 and cfg["global_batch"] == 8 and cfg["prefill_len"] == 300 and cfg["prompt_len"] == 70
-    for side in ("melizen", "llama_of_equal_size"):
+    for side in (arch, "llama_of_equal_size"):
         assert set(d[side]) == {"prefill_ms", "prefill_tok_s", "decode_ms_per_step", "decode_tok_s"}
         assert all(v > 0 for v in d[side].values())
-    assert d["value"] == d["melizen"]["decode_tok_s"] and d["ms_per_step"] == d["melizen"]["decode_ms_per_step"]
-    assert abs(d["melizen_over_llama"]["decode_step_time"]
-               - d["melizen"]["decode_ms_per_step"] / d["llama_of_equal_size"]["decode_ms_per_step"]) < 2e-3
+    assert d["value"] == d[arch]["decode_tok_s"] and d["ms_per_step"] == d[arch]["decode_ms_per_step"]
+    assert abs(d[f"{arch}_over_llama"]["decode_step_time"]
+               - d[arch]["decode_ms_per_step"] / d["llama_of_equal_size"]["decode_ms_per_step"]) < 2e-3
