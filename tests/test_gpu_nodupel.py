@@ -557,3 +557,97 @@ def test_the_trace_runner_replays_a_model_of_this_design(tmp_path):
     close(np.concatenate(got["c"]), ref["c"], "float32", "the shorter of a batch")
     close(np.concatenate(got["a"]), ref["a"][69:90], "float32", "the longer of a batch")
     rp.close()
+
+
+# ----------------------------------------------------------------- seeded random configurations
+def random_config(seed):
+    """Sizes, counts, order of layers, windows and constants drawn from a seed: what no hand-made configuration
+    happened to combine."""
+    rng = np.random.default_rng([seed, 99])
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    width = pick([40, 64, 72, 90, 128, 200])
+    n_layers = int(rng.integers(2, 6))
+    layers = []
+    for i in range(n_layers):
+        ff = pick([None, 48, 100, 192, 256])
+        mlp = None if ff is None else {"kind": "dense", "ff": ff}
+        if rng.random() < 0.35:
+            layers.append({"type": "mingru", "mixer": {"width": pick([16, 50, 64, 136, 200])}, "mlp": mlp})
+            continue
+        heads = pick([1, 2, 3, 4, 6, 8])
+        kv = pick([k for k in (1, 2, 3, 4, 6, 8) if heads % k == 0])
+        dim, vdim = pick([8, 16, 24, 32, 40, 64, 96, 128]), pick([8, 16, 24, 32, 48, 64, 96, 128])
+        dims = pick([d for d in (2, 4, 8, 16, 24, 32, 64, 96, 128) if d <= dim])
+        rot = {"base": pick([100.0, 10000.0, 500000.0]), "dims": dims}
+        if rng.random() < 0.5:
+            rot["scaling"] = {"factor": pick([1.5, 2.0, 8.0])}
+        left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": float(pick([0.1, 0.2, dim ** -0.5])), "rot": rot}
+        if rng.random() < 0.8:
+            left["mask"] = {"size": pick([1, 2, 7, 31, 32, 64, 65, 100, 150]), "keep_first": pick([0, 1, 3, 16, 64, 65, 80])}
+        layers.append({"type": "parallel", "mlp": mlp,
+                       "mixer": {"left": left, "right": {"heads": pick([1, 2, 3, 4]), "dim": pick([8, 16, 20, 32, 48, 64, 80])}}})
+    if not any(l["type"] == "parallel" for l in layers):
+        layers[0], layers[-1] = layers[-1], layers[0]
+    cfg = {"architecture": "Nodupel", "vocab": int(rng.integers(50, 700)), "width": width, "norm": {"eps": pick([1e-5, 1e-6])},
+           "residual_mult": float(pick([0.25, 0.5, 0.9, 1.0, 1.2])),
+           "embedding": {"scale": float(pick([1.0, 3.0, width ** 0.5])),
+                         "bigram": {"buckets": int(rng.integers(1, 2000)), "mul_prev": int(rng.integers(1, 10 ** 6)),
+                                    "mul_cur": int(rng.integers(1, 10 ** 6))}},
+           "layers": layers}
+    if rng.random() < 0.7:
+        cfg["logit_softcap"] = float(pick([5.0, 30.0, 50.0]))
+    if rng.random() < 0.7:
+        start = int(rng.integers(0, n_layers))
+        cfg["loop"] = {"start": start, "stop": int(rng.integers(start + 1, n_layers + 1)), "times": int(rng.integers(1, 4))}
+    return cfg, int(rng.integers(1, 40))
+
+
+def close_mostly(got, ref, dtype, what):
+    """32-bit: every row within the bound. bfloat16: a drawn configuration may run nine layers over a width of 40, where
+    single rows gather more rounding than the hand-made models' bound allows for: at most one row in fifty beyond the
+    bound, none beyond twice the bound (a fault moves whole runs of rows by many times that)."""
+    if dtype == "float32":
+        return close(got, ref, dtype, what)
+    e = row_errors(got, ref)
+    assert (e > 2 * TOL[dtype]).sum() == 0 and (e > TOL[dtype]).sum() <= max(1, len(e) // 50), \
+        f"{what}: {int((e > TOL[dtype]).sum())} of {len(e)} rows over {TOL[dtype]}, the worst {e.max():.3e}"
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_seeded_random_configurations(seed, tmp_path):
+    import json
+    import os
+    from safetensors.torch import save_file
+    from gpullama3_java_amd.engine import Engine
+    cfg, rank = random_config(seed)
+    W = P.make_weights(cfg, seed, rank)
+    save_file({k: torch.tensor(v).to(torch.bfloat16).contiguous() for k, v in W.items()}, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    rng = np.random.default_rng([seed, 7])
+    prompts = [rng.integers(0, cfg["vocab"], size=n).tolist() for n in (172, 1, 40)]
+    refs = [P.forward(cfg, W, p) for p in prompts]
+    for dtype in DTYPES:
+        eng = Engine.from_folder(str(tmp_path), dtype=dtype, max_tokens=1024, n_slots=4)
+        # whole; the last 40 tokens one by one; three unequal requests in one batch, then together token by token
+        s = eng.take_slot()
+        close_mostly(eng.step([(s, prompts[0])], want="all").cpu().numpy(), refs[0], dtype, f"seed {seed} whole")
+        eng.give_back_slot(s)
+        s = eng.take_slot()
+        rows = [eng.step([(s, prompts[0][:132])], want="all").cpu().numpy()]
+        for t in prompts[0][132:]:
+            rows.append(eng.step([(s, [t])]).cpu().numpy())
+        close_mostly(np.concatenate(rows), refs[0], dtype, f"seed {seed} decoded")
+        eng.give_back_slot(s)
+        slots = [eng.take_slot() for _ in prompts]
+        cut = [150, 1, 20]
+        got = eng.step([(slots[i], prompts[i][:cut[i]]) for i in range(3)], want="all").cpu().numpy()
+        lo = 0
+        for i in range(3):
+            close_mostly(got[lo:lo + cut[i]], refs[i][:cut[i]], dtype, f"seed {seed} batch prompt {i}")
+            lo += cut[i]
+        for step in range(20):
+            live = [i for i in range(3) if cut[i] + step < len(prompts[i])]
+            got = eng.step([(slots[i], [prompts[i][cut[i] + step]]) for i in live]).cpu().numpy()
+            for r, i in enumerate(live):
+                close_mostly(got[r:r + 1], refs[i][cut[i] + step:cut[i] + step + 1], dtype, f"seed {seed} batch step {step} request {i}")
+        del eng
